@@ -1,0 +1,103 @@
+"""ctypes bindings of the C-ABI kernel layer (include/trtamd_bert_kernels.h).
+
+Functions take raw device addresses (ints) — e.g. ``torch.Tensor.data_ptr()`` — and a stream
+handle; nothing here touches torch.  ``check`` turns a non-zero status into an exception carrying
+``trtamd_last_error()``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+from . import load_library
+
+c_p = C.c_void_p
+i32 = C.c_int32
+i64 = C.c_int64
+u32 = C.c_uint32
+f32 = C.c_float
+
+
+class FmhaParams(C.Structure):
+    """struct trtamd_fmha_params."""
+    _fields_ = [
+        ("qkv_ptr", c_p), ("packed_mask_ptr", c_p), ("o_ptr", c_p),
+        ("qkv_stride_in_bytes", i64), ("packed_mask_stride_in_bytes", i64), ("o_stride_in_bytes", i64),
+        ("b", i32), ("h", i32), ("s", i32), ("d", i32),
+        ("scale_bmm1", u32), ("scale_softmax", u32), ("scale_bmm2", u32),
+        ("enable_i2f_trick", i32),
+        ("cu_seqlens", c_p),
+        ("interleaved", i32), ("use_int8_scale_max", i32),
+        ("warps_m", i32), ("warps_n", i32),
+    ]
+
+
+_SIGS = {
+    "trtamd_version": (C.c_int, []),
+    "trtamd_last_error": (C.c_char_p, []),
+    "trtamd_skip_layer_norm_fp32": (C.c_int, [c_p, i32, i64, c_p, c_p, c_p, c_p, c_p, c_p]),
+    "trtamd_skip_layer_norm_fp16": (C.c_int, [c_p, i32, i64, c_p, c_p, c_p, c_p, c_p, c_p]),
+    "trtamd_skip_layer_norm_dqq": (C.c_int, [c_p, i32, i64, c_p, c_p, c_p, c_p, c_p, c_p, f32, f32, f32]),
+    "trtamd_skipln_interleaved_small_hface": (C.c_int, [c_p, i32, i32, c_p, c_p, c_p, c_p, c_p, f32, f32, f32]),
+    "trtamd_skipln_interleaved_large_hface": (C.c_int, [c_p, i32, i32, c_p, c_p, c_p, c_p, c_p, f32, f32, f32]),
+    "trtamd_skipln_interleaved_small_mtron": (C.c_int, [c_p, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, f32, f32, f32,
+                                                        f32]),
+    "trtamd_skipln_interleaved_large_mtron": (C.c_int, [c_p, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, f32, f32, f32,
+                                                        f32]),
+    "trtamd_emb_layer_norm_fp32": (C.c_int, [c_p, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, i32, i32, c_p]),
+    "trtamd_emb_layer_norm_fp16": (C.c_int, [c_p, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, i32, i32, c_p]),
+    "trtamd_emb_layer_norm_hface_fp32": (C.c_int, [c_p, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, i32, i32,
+                                                   c_p]),
+    "trtamd_emb_layer_norm_hface_fp16": (C.c_int, [c_p, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, i32, i32,
+                                                   c_p]),
+    "trtamd_emb_layer_norm_mtron_fp32": (C.c_int, [c_p, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, i32, i32,
+                                                   c_p, c_p]),
+    "trtamd_emb_layer_norm_mtron_fp16": (C.c_int, [c_p, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, i32, i32,
+                                                   c_p, c_p]),
+    "trtamd_compute_mask_idx": (C.c_int, [c_p, i32, i32, c_p, c_p]),
+    "trtamd_convert_mask": (C.c_int, [u32, u32, u32, u32, u32, c_p, c_p, c_p]),
+    "trtamd_scaled_softmax_fp32": (C.c_int, [c_p, i32, i32, i32, f32, c_p, c_p, c_p]),
+    "trtamd_scaled_softmax_fp16": (C.c_int, [c_p, i32, i32, i32, f32, c_p, c_p, c_p]),
+    "trtamd_unfused_mha_workspace_size": (C.c_size_t, [i32, i32, i32, i32]),
+    "trtamd_unfused_mha": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p, c_p]),
+    "trtamd_fused_mha_run": (C.c_int, [c_p, i32, C.POINTER(FmhaParams)]),
+    "trtamd_fused_mha_run_debug": (C.c_int, [c_p, i32, C.POINTER(FmhaParams), c_p, c_p]),
+    "trtamd_fused_mha_is_valid": (C.c_int, [i32, i32, i32]),
+    "trtamd_zero_padding_2d": (C.c_int, [c_p, i32, c_p, i32, i32, c_p]),
+}
+
+# Entry points declared in include/trtamd_bert_kernels.h (the debug hook is extra).
+HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug"]
+
+
+class TrtAmdError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+class _Api:
+    def __init__(self):
+        self._lib = load_library()
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(self._lib, name)
+            fn.restype = res
+            fn.argtypes = args
+            setattr(self, name[len("trtamd_"):], fn)
+
+    def last_error_str(self) -> str:
+        return (self.last_error() or b"").decode()
+
+    def check(self, status: int) -> None:
+        if status != 0:
+            raise TrtAmdError(status, self.last_error_str())
+
+
+_api = None
+
+
+def api() -> _Api:
+    global _api
+    if _api is None:
+        _api = _Api()
+    return _api

@@ -1,0 +1,46 @@
+// Host-side helpers of the C-ABI layer: per-thread error text and launch checking.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "trtamd_bert_kernels.h"
+
+namespace trtamd
+{
+
+// Stores a printf-style message retrievable through trtamd_last_error() and returns `status`.
+int set_error(int status, char const* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Status of the launch that was just issued (hipPeekAtLastError semantics of the reference's
+// PLUGIN_CHECK(cudaPeekAtLastError()) without terminating the process).
+inline int check_launch(char const* what)
+{
+    hipError_t const e = hipGetLastError();
+    if (e != hipSuccess)
+    {
+        return set_error(TRTAMD_STATUS_FAILURE, "%s: %s", what, hipGetErrorString(e));
+    }
+    return TRTAMD_STATUS_SUCCESS;
+}
+
+inline hipStream_t as_stream(trtamd_stream_t s)
+{
+    return reinterpret_cast<hipStream_t>(s);
+}
+
+inline bool aligned16(void const* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+template <typename T>
+constexpr T ceil_div(T a, T b)
+{
+    return (a + b - 1) / b;
+}
+
+} // namespace trtamd

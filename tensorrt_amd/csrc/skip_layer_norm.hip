@@ -1,0 +1,705 @@
+// SkipLayerNorm kernels for gfx950: residual (+bias) + LayerNorm on rows of `ld` elements.
+//
+// All variants are HBM-bound streams.  Common shape: one 64-lane wavefront owns whole rows (or,
+// for the 32-interleaved INT8 layout, 8 adjacent tokens), keeps the row in registers between the
+// statistics and the normalisation (one read, one write per element), reduces with lane shuffles
+// only (no LDS, no barrier on the data path) and issues every global load of its rows before the
+// first arithmetic so that several KB per wave are in flight.
+//
+// Replaces plugin/skipLayerNormPlugin/skipLayerNormKernel.cu,
+// plugin/skipLayerNormPlugin/skipLayerNormInt8InterleavedKernelHFace.cu and
+// plugin/skipLayerNormPlugin/skipLayerNormInt8InterleavedKernelMTron.cu of the reference.
+#include "device_utils.hpp"
+#include "host_utils.hpp"
+
+namespace trtamd
+{
+namespace
+{
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWaveSize;
+
+template <typename T>
+struct Vec16
+{
+    static constexpr int kN = 16 / sizeof(T);
+    union
+    {
+        u32x4 u;
+        T e[kN];
+    };
+};
+
+// ------------------------------------------------------------------------------------------
+// FP32 / FP16 rows, ld a multiple of the 16-byte vector width: register-resident rows.
+// The residual sum is formed in T like the reference (skipLayerNormKernel.cu:121-134);
+// statistics are a Welford/Chan merge in binary32; epsilon is the caller's.
+// ------------------------------------------------------------------------------------------
+template <typename T, int NV, int R, bool HAS_BIAS>
+__global__ __launch_bounds__(kBlock) void skipln_rows_kernel(int const ld, int64_t const rows, T const* __restrict__ in,
+    T const* __restrict__ skip, T const* __restrict__ beta, T const* __restrict__ gamma, T const* __restrict__ bias,
+    T* __restrict__ out, float const eps)
+{
+    constexpr int VPT = Vec16<T>::kN;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int64_t const wave = (int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    int64_t const row0 = wave * R;
+    if (row0 >= rows)
+    {
+        return;
+    }
+    int const nvec = ld / VPT;
+
+    Vec16<T> xin[R][NV], xsk[R][NV];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            int const vi = lane + kWaveSize * j;
+            bool const ok = vi < nvec && row0 + r < rows;
+            int64_t const off = (row0 + r) * ld + (int64_t) vi * VPT;
+            xin[r][j].u = ok ? *reinterpret_cast<u32x4 const*>(in + off) : u32x4{0, 0, 0, 0};
+            xsk[r][j].u = ok ? *reinterpret_cast<u32x4 const*>(skip + off) : u32x4{0, 0, 0, 0};
+        }
+    }
+    Vec16<T> g[NV], b[NV], bs[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+    {
+        int const vi = lane + kWaveSize * j;
+        bool const ok = vi < nvec;
+        g[j].u = ok ? *reinterpret_cast<u32x4 const*>(gamma + vi * VPT) : u32x4{0, 0, 0, 0};
+        b[j].u = ok ? *reinterpret_cast<u32x4 const*>(beta + vi * VPT) : u32x4{0, 0, 0, 0};
+        if (HAS_BIAS)
+        {
+            bs[j].u = ok ? *reinterpret_cast<u32x4 const*>(bias + vi * VPT) : u32x4{0, 0, 0, 0};
+        }
+    }
+
+    float const rld = 1.f / (float) ld;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        if (row0 + r >= rows)
+        {
+            break; // wave-uniform
+        }
+        float v[NV][VPT];
+        float sum = 0.f;
+        float cnt = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            bool const ok = lane + kWaveSize * j < nvec;
+#pragma unroll
+            for (int k = 0; k < VPT; ++k)
+            {
+                T t = xin[r][j].e[k] + xsk[r][j].e[k];
+                if (HAS_BIAS)
+                {
+                    t = t + bs[j].e[k];
+                }
+                v[j][k] = (float) t;
+                sum += ok ? v[j][k] : 0.f;
+            }
+            cnt += ok ? (float) VPT : 0.f;
+        }
+        Welford w;
+        w.n = cnt;
+        w.mean = cnt > 0.f ? sum / cnt : 0.f;
+        w.m2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            bool const ok = lane + kWaveSize * j < nvec;
+#pragma unroll
+            for (int k = 0; k < VPT; ++k)
+            {
+                float const dlt = v[j][k] - w.mean;
+                w.m2 += ok ? dlt * dlt : 0.f;
+            }
+        }
+        w = group_welford<kWaveSize>(w);
+        float const mu = w.mean;
+        float const rsigma = rsqrtf(w.m2 * rld + eps);
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            int const vi = lane + kWaveSize * j;
+            if (vi < nvec)
+            {
+                Vec16<T> y;
+#pragma unroll
+                for (int k = 0; k < VPT; ++k)
+                {
+                    y.e[k] = (T) ((float) g[j].e[k] * (v[j][k] - mu) * rsigma + (float) b[j].e[k]);
+                }
+                *reinterpret_cast<u32x4*>(out + (row0 + r) * ld + (int64_t) vi * VPT) = y.u;
+            }
+        }
+    }
+}
+
+// Any ld (odd sizes, ld <= 32, very long rows): one wave per row, three L2-resident sweeps.
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(kBlock) void skipln_generic_kernel(int const ld, int64_t const rows,
+    T const* __restrict__ in, T const* __restrict__ skip, T const* __restrict__ beta, T const* __restrict__ gamma,
+    T const* __restrict__ bias, T* __restrict__ out, float const eps)
+{
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int64_t const row = (int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (row >= rows)
+    {
+        return;
+    }
+    T const* pi = in + row * ld;
+    T const* ps = skip + row * ld;
+    auto value = [&](int i) -> float {
+        T t = pi[i] + ps[i];
+        if (HAS_BIAS)
+        {
+            t = t + bias[i];
+        }
+        return (float) t;
+    };
+    float sum = 0.f;
+    for (int i = lane; i < ld; i += kWaveSize)
+    {
+        sum += value(i);
+    }
+    float const mu = wave_sum(sum) / (float) ld;
+    float m2 = 0.f;
+    for (int i = lane; i < ld; i += kWaveSize)
+    {
+        float const dlt = value(i) - mu;
+        m2 += dlt * dlt;
+    }
+    float const rsigma = rsqrtf(wave_sum(m2) / (float) ld + eps);
+    for (int i = lane; i < ld; i += kWaveSize)
+    {
+        out[row * ld + i] = (T) ((float) gamma[i] * (value(i) - mu) * rsigma + (float) beta[i]);
+    }
+}
+
+template <typename T, int NV, int R>
+int launch_rows(hipStream_t stream, int ld, int64_t rows, T const* in, T const* skip, T const* beta, T const* gamma,
+    T const* bias, T* out, float eps)
+{
+    int64_t const waves = ceil_div<int64_t>(rows, R);
+    dim3 const grid((unsigned) ceil_div<int64_t>(waves, kWavesPerBlock));
+    if (bias)
+    {
+        hipLaunchKernelGGL((skipln_rows_kernel<T, NV, R, true>), grid, dim3(kBlock), 0, stream, ld, rows, in, skip, beta,
+            gamma, bias, out, eps);
+    }
+    else
+    {
+        hipLaunchKernelGGL((skipln_rows_kernel<T, NV, R, false>), grid, dim3(kBlock), 0, stream, ld, rows, in, skip,
+            beta, gamma, bias, out, eps);
+    }
+    return check_launch("skipln_rows_kernel");
+}
+
+template <typename T>
+int skip_layer_norm(hipStream_t stream, int32_t ld, int64_t n, T const* in, T const* skip, T const* beta,
+    T const* gamma, T* out, T const* bias, float epsT)
+{
+    if (ld <= 0 || n < 0 || n % ld != 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNorm: n (%lld) must be a multiple of ld (%d)",
+            (long long) n, ld);
+    }
+    if (n == 0)
+    {
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    if (!in || !skip || !beta || !gamma || !out)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNorm: null tensor pointer");
+    }
+    int64_t const rows = n / ld;
+    // The reference adds numeric_limits<T>::epsilon() only in its vectorised kernel, which it
+    // selects for ld in {768,1024} (skipLayerNormKernel.cu:267-276, 149).
+    float const eps = (ld == 768 || ld == 1024) ? epsT : 0.f;
+    constexpr int VPT = 16 / (int) sizeof(T);
+    bool const vec_ok = ld % VPT == 0 && ld > 32 && aligned16(in) && aligned16(skip) && aligned16(out)
+        && aligned16(beta) && aligned16(gamma) && (!bias || aligned16(bias));
+    int const nv = vec_ok ? ceil_div(ld / VPT, kWaveSize) : 0;
+    if (vec_ok && nv == 1)
+    {
+        return launch_rows<T, 1, 4>(stream, ld, rows, in, skip, beta, gamma, bias, out, eps);
+    }
+    if (vec_ok && nv == 2)
+    {
+        return launch_rows<T, 2, 2>(stream, ld, rows, in, skip, beta, gamma, bias, out, eps);
+    }
+    if (vec_ok && nv <= 4)
+    {
+        return launch_rows<T, 4, 1>(stream, ld, rows, in, skip, beta, gamma, bias, out, eps);
+    }
+    if (vec_ok && nv <= 8)
+    {
+        return launch_rows<T, 8, 1>(stream, ld, rows, in, skip, beta, gamma, bias, out, eps);
+    }
+    dim3 const grid((unsigned) ceil_div<int64_t>(rows, kWavesPerBlock));
+    if (bias)
+    {
+        hipLaunchKernelGGL((skipln_generic_kernel<T, true>), grid, dim3(kBlock), 0, stream, ld, rows, in, skip, beta,
+            gamma, bias, out, eps);
+    }
+    else
+    {
+        hipLaunchKernelGGL((skipln_generic_kernel<T, false>), grid, dim3(kBlock), 0, stream, ld, rows, in, skip, beta,
+            gamma, bias, out, eps);
+    }
+    return check_launch("skipln_generic_kernel");
+}
+
+// ------------------------------------------------------------------------------------------
+// INT8 rows, linear layout (skiplnDQQ, skipLayerNormKernel.cu:43-106): each lane owns 16
+// consecutive channels of a row, a wave owns R rows.  v = dqIn*in + dqSkip*skip (+bias) in
+// binary32, Welford statistics, epsilon 2^-10, out = sat8(rne(y * qScale)).
+// ------------------------------------------------------------------------------------------
+template <int R, bool HAS_BIAS>
+__global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_t const rows,
+    int8_t const* __restrict__ in, int8_t const* __restrict__ skip, f16 const* __restrict__ beta,
+    f16 const* __restrict__ gamma, f16 const* __restrict__ bias, int8_t* __restrict__ out, float const dqIn,
+    float const dqSkip, float const qScale)
+{
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int64_t const wave = (int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    int64_t const row0 = wave * R;
+    if (row0 >= rows)
+    {
+        return;
+    }
+    bool const lane_ok = lane * 16 < ld;
+    u32x4 xi[R], xs[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        bool const ok = lane_ok && row0 + r < rows;
+        int64_t const off = (row0 + r) * ld + lane * 16;
+        xi[r] = ok ? *reinterpret_cast<u32x4 const*>(in + off) : u32x4{0, 0, 0, 0};
+        xs[r] = ok ? *reinterpret_cast<u32x4 const*>(skip + off) : u32x4{0, 0, 0, 0};
+    }
+    Vec16<f16> g[2], b[2], bs[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+    {
+        int const c = lane * 16 + h * 8;
+        g[h].u = lane_ok ? *reinterpret_cast<u32x4 const*>(gamma + c) : u32x4{0, 0, 0, 0};
+        b[h].u = lane_ok ? *reinterpret_cast<u32x4 const*>(beta + c) : u32x4{0, 0, 0, 0};
+        if (HAS_BIAS)
+        {
+            bs[h].u = lane_ok ? *reinterpret_cast<u32x4 const*>(bias + c) : u32x4{0, 0, 0, 0};
+        }
+    }
+    float const rld = 1.f / (float) ld;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+    {
+        if (row0 + r >= rows)
+        {
+            break;
+        }
+        float v[16];
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+        {
+            float x = dqIn * i8_to_f32(xi[r][k >> 2], k & 3) + dqSkip * i8_to_f32(xs[r][k >> 2], k & 3);
+            if (HAS_BIAS)
+            {
+                x += (float) bs[k >> 3].e[k & 7];
+            }
+            v[k] = x;
+            sum += x;
+        }
+        Welford w;
+        w.n = lane_ok ? 16.f : 0.f;
+        w.mean = sum * (1.f / 16.f);
+        w.m2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+        {
+            float const dlt = v[k] - w.mean;
+            w.m2 += dlt * dlt;
+        }
+        if (!lane_ok)
+        {
+            w.mean = 0.f;
+            w.m2 = 0.f;
+        }
+        w = group_welford<kWaveSize>(w);
+        float const mu = w.mean;
+        float const rsigma = rsqrtf(w.m2 * rld + 0.0009765625f);
+        if (lane_ok)
+        {
+            u32x4 o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                int p[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                {
+                    int const c = q * 4 + k;
+                    float const y = (float) g[c >> 3].e[c & 7] * (v[c] - mu) * rsigma + (float) b[c >> 3].e[c & 7];
+                    p[k] = sat8_rne(y * qScale);
+                }
+                o[q] = pack_i8x4(p[0], p[1], p[2], p[3]);
+            }
+            *reinterpret_cast<u32x4*>(out + (row0 + r) * ld + lane * 16) = o;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// INT8, 32-interleaved layout [ld/32][total][32] (TensorFormat::kCHW32 of a [1,ld,total,1]
+// tensor).  A wave owns 8 adjacent tokens: lane = (sub, tok, half) with sub = lane/16 selecting
+// one of 4 channel groups per step, tok = (lane%16)/2, half = lane%2 selecting 16 of the group's
+// 32 channels.  One 16-byte load per lane therefore covers 4 channel groups x 256 contiguous
+// bytes.  Statistics come from exact integer dot products (sum in, sum skip, sum in^2, sum
+// in*skip, sum skip^2) combined in binary64, so mean and variance carry no accumulation error.
+// gamma*qScale and beta*qScale are staged once per workgroup in LDS as binary32.
+// ------------------------------------------------------------------------------------------
+template <int G, bool PRELN>
+__global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const total, int8_t const* __restrict__ in,
+    int8_t const* __restrict__ skip, f16 const* __restrict__ beta, f16 const* __restrict__ gamma,
+    int8_t* __restrict__ out, int8_t* __restrict__ preln, float const dqIn, float const dqSkip, float const qScale,
+    float const qSkipScale, float const eps, float const prelnMin)
+{
+    constexpr int LD = G * 32;
+    constexpr int NI = G / 4;
+    constexpr bool RESIDENT = NI <= 8;
+    __shared__ float sGamma[LD];
+    __shared__ float sBeta[LD];
+    for (int i = threadIdx.x; i < LD; i += kBlock)
+    {
+        sGamma[i] = (float) gamma[i] * qScale;
+        sBeta[i] = (float) beta[i] * qScale;
+    }
+    __syncthreads();
+
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const sub = lane >> 4;
+    int const tok = (lane & 15) >> 1;
+    int const hf = lane & 1;
+    int64_t const t = ((int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * 8 + tok;
+    bool const valid = t < total;
+    int64_t const groupStride = (int64_t) total * 32;
+    int64_t const base = (int64_t) sub * groupStride + t * 32 + hf * 16;
+
+    u32x4 xi[RESIDENT ? NI : 1], xs[RESIDENT ? NI : 1];
+    int sIn = 0, sSk = 0, sII = 0, sIS = 0, sSS = 0;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+    {
+        u32x4 a = {0, 0, 0, 0}, s = {0, 0, 0, 0};
+        if (valid)
+        {
+            a = *reinterpret_cast<u32x4 const*>(in + base + (int64_t) i * 4 * groupStride);
+            s = *reinterpret_cast<u32x4 const*>(skip + base + (int64_t) i * 4 * groupStride);
+        }
+        if (RESIDENT)
+        {
+            xi[i] = a;
+            xs[i] = s;
+        }
+        else
+        {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                sIn = __builtin_amdgcn_sdot4((int) a[q], 0x01010101, sIn, false);
+                sSk = __builtin_amdgcn_sdot4((int) s[q], 0x01010101, sSk, false);
+                sII = __builtin_amdgcn_sdot4((int) a[q], (int) a[q], sII, false);
+                sIS = __builtin_amdgcn_sdot4((int) a[q], (int) s[q], sIS, false);
+                sSS = __builtin_amdgcn_sdot4((int) s[q], (int) s[q], sSS, false);
+            }
+        }
+    }
+    if (RESIDENT)
+    {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+        {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                sIn = __builtin_amdgcn_sdot4((int) xi[i][q], 0x01010101, sIn, false);
+                sSk = __builtin_amdgcn_sdot4((int) xs[i][q], 0x01010101, sSk, false);
+                sII = __builtin_amdgcn_sdot4((int) xi[i][q], (int) xi[i][q], sII, false);
+                sIS = __builtin_amdgcn_sdot4((int) xi[i][q], (int) xs[i][q], sIS, false);
+                sSS = __builtin_amdgcn_sdot4((int) xs[i][q], (int) xs[i][q], sSS, false);
+            }
+        }
+    }
+    // the 8 lanes of a token differ in bit 0 (half) and bits 4,5 (sub)
+#pragma unroll
+    for (int m : {1, 16, 32})
+    {
+        sIn += __shfl_xor(sIn, m, kWaveSize);
+        sSk += __shfl_xor(sSk, m, kWaveSize);
+        sII += __shfl_xor(sII, m, kWaveSize);
+        sIS += __shfl_xor(sIS, m, kWaveSize);
+        sSS += __shfl_xor(sSS, m, kWaveSize);
+    }
+    double const dIn = (double) dqIn, dSk = (double) dqSkip;
+    double const mean = (dIn * sIn + dSk * sSk) * (1.0 / LD);
+    double const ex2 = (dIn * dIn * sII + 2.0 * dIn * dSk * sIS + dSk * dSk * sSS) * (1.0 / LD);
+    float const var = (float) (ex2 - mean * mean);
+    float const rsigma = rsqrtf(fmaxf(var, 0.f) + eps);
+    // bytes are read as unsigned after flipping the sign bit: u = x + 128
+    float const a1 = dqIn * rsigma;
+    float const a2 = dqSkip * rsigma;
+    float const c1 = (float) ((-128.0 * (dIn + dSk) - mean) * (double) rsigma);
+    float const p1 = dqIn * qSkipScale;
+    float const p2 = dqSkip * qSkipScale;
+    float const pc = -128.f * (dqIn + dqSkip) * qSkipScale;
+    constexpr float kMagic = 12582912.f; // 1.5 * 2^23: the sum's low mantissa byte is rne(x) in two's complement
+
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+    {
+        u32x4 a, s;
+        if (RESIDENT)
+        {
+            a = xi[i];
+            s = xs[i];
+        }
+        else
+        {
+            a = u32x4{0, 0, 0, 0};
+            s = u32x4{0, 0, 0, 0};
+            if (valid)
+            {
+                a = *reinterpret_cast<u32x4 const*>(in + base + (int64_t) i * 4 * groupStride);
+                s = *reinterpret_cast<u32x4 const*>(skip + base + (int64_t) i * 4 * groupStride);
+            }
+        }
+        int const ch = (i * 4 + sub) * 32 + hf * 16;
+        u32x4 o, po;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            uint32_t const ua = a[q] ^ 0x80808080u;
+            uint32_t const us = s[q] ^ 0x80808080u;
+            f32x4 const gq = *reinterpret_cast<f32x4 const*>(&sGamma[ch + q * 4]);
+            f32x4 const bq = *reinterpret_cast<f32x4 const*>(&sBeta[ch + q * 4]);
+            uint32_t yb[4], pb[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                float const fa = (float) ((ua >> (8 * k)) & 0xffu);
+                float const fs = (float) ((us >> (8 * k)) & 0xffu);
+                float const nrm = fmaf(fa, a1, fmaf(fs, a2, c1));
+                float y = fmaf(gq[k], nrm, bq[k]);
+                y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
+                yb[k] = __float_as_uint(y + kMagic);
+                if (PRELN)
+                {
+                    float p = fmaf(fa, p1, fmaf(fs, p2, pc));
+                    p = __builtin_amdgcn_fmed3f(p, prelnMin, 127.f);
+                    pb[k] = __float_as_uint(p + kMagic);
+                }
+            }
+            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+            o[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            if (PRELN)
+            {
+                uint32_t const plo = __builtin_amdgcn_perm(pb[1], pb[0], 0x0c0c0400u);
+                uint32_t const phi = __builtin_amdgcn_perm(pb[3], pb[2], 0x0c0c0400u);
+                po[q] = __builtin_amdgcn_perm(phi, plo, 0x05040100u);
+            }
+        }
+        if (valid)
+        {
+            *reinterpret_cast<u32x4*>(out + base + (int64_t) i * 4 * groupStride) = o;
+            if (PRELN)
+            {
+                *reinterpret_cast<u32x4*>(preln + base + (int64_t) i * 4 * groupStride) = po;
+            }
+        }
+    }
+}
+
+template <int G>
+int launch_interleaved(hipStream_t stream, int32_t total, int8_t const* in, int8_t const* skip, f16 const* beta,
+    f16 const* gamma, int8_t* out, int8_t* preln, float dqIn, float dqSkip, float qScale, float qSkipScale, float eps,
+    float prelnMin)
+{
+    dim3 const grid((unsigned) ceil_div(total, 8 * kWavesPerBlock));
+    if (preln)
+    {
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, true>), grid, dim3(kBlock), 0, stream, total, in, skip, beta,
+            gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
+    }
+    else
+    {
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, false>), grid, dim3(kBlock), 0, stream, total, in, skip, beta,
+            gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
+    }
+    return check_launch("skipln_interleaved_kernel");
+}
+
+// small: epsilon = binary16 epsilon, preln clipped to +-127; large: binary32 epsilon, preln
+// saturated to [-128,127].  maxLdSet: which ld values the reference launcher accepts.
+int skipln_interleaved(hipStream_t stream, bool large, bool mtron, int32_t ld, int32_t total, int8_t const* in,
+    int8_t const* skip, f16 const* beta, f16 const* gamma, int8_t* out, int8_t* preln, float dqIn, float dqSkip,
+    float qScale, float qSkipScale)
+{
+    bool const base_ok = ld == 768 || ld == 1024;
+    bool const wide_ok = !large && mtron && (ld == 1536 || ld == 2048 || ld == 3072 || ld == 4096);
+    if (!base_ok && !wide_ok)
+    {
+        return set_error(TRTAMD_STATUS_FAILURE, "SkipLayerNormDQQ - FATAL: unsupported hidden layer size: %d", ld);
+    }
+    if (total < 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNorm interleaved: negative token count");
+    }
+    if (total == 0)
+    {
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    if (!in || !skip || !beta || !gamma || !out || (mtron && !preln))
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNorm interleaved: null tensor pointer");
+    }
+    if (!aligned16(in) || !aligned16(skip) || !aligned16(out) || (mtron && !aligned16(preln)))
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNorm interleaved: tensors must be 16-byte aligned");
+    }
+    float const eps = large ? 1.1920928955078125e-07f : 0.0009765625f;
+    float const pmin = large ? -128.f : -127.f;
+    int8_t* pre = mtron ? preln : nullptr;
+    switch (ld)
+    {
+    case 768:
+        return launch_interleaved<24>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
+            eps, pmin);
+    case 1024:
+        return launch_interleaved<32>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
+            eps, pmin);
+    case 1536:
+        return launch_interleaved<48>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
+            eps, pmin);
+    case 2048:
+        return launch_interleaved<64>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
+            eps, pmin);
+    case 3072:
+        return launch_interleaved<96>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
+            eps, pmin);
+    default:
+        return launch_interleaved<128>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale,
+            qSkipScale, eps, pmin);
+    }
+}
+
+} // namespace
+} // namespace trtamd
+
+using namespace trtamd;
+
+extern "C" int trtamd_skip_layer_norm_fp32(trtamd_stream_t stream, int32_t ld, int64_t n, float const* input,
+    float const* skip, float const* beta, float const* gamma, float* output, float const* bias)
+{
+    return skip_layer_norm<float>(as_stream(stream), ld, n, input, skip, beta, gamma, output, bias,
+        1.1920928955078125e-07f);
+}
+
+extern "C" int trtamd_skip_layer_norm_fp16(trtamd_stream_t stream, int32_t ld, int64_t n, trtamd_half_t const* input,
+    trtamd_half_t const* skip, trtamd_half_t const* beta, trtamd_half_t const* gamma, trtamd_half_t* output,
+    trtamd_half_t const* bias)
+{
+    return skip_layer_norm<f16>(as_stream(stream), ld, n, reinterpret_cast<f16 const*>(input),
+        reinterpret_cast<f16 const*>(skip), reinterpret_cast<f16 const*>(beta), reinterpret_cast<f16 const*>(gamma),
+        reinterpret_cast<f16*>(output), reinterpret_cast<f16 const*>(bias), 0.0009765625f);
+}
+
+extern "C" int trtamd_skip_layer_norm_dqq(trtamd_stream_t stream, int32_t ld, int64_t n, int8_t const* input,
+    int8_t const* skip, trtamd_half_t const* beta, trtamd_half_t const* gamma, int8_t* output,
+    trtamd_half_t const* bias, float dqScaleIn, float dqScaleSkip, float qScale)
+{
+    if (ld <= 0 || n < 0 || n % ld != 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNormDQQ: n (%lld) must be a multiple of ld (%d)",
+            (long long) n, ld);
+    }
+    if (ld != 768 && ld != 1024)
+    {
+        return set_error(TRTAMD_STATUS_FAILURE, "SkipLayerNormDQQ - FATAL: unsupported hidden layer size: %d", ld);
+    }
+    if (n == 0)
+    {
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    if (!input || !skip || !beta || !gamma || !output)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNormDQQ: null tensor pointer");
+    }
+    if (!aligned16(input) || !aligned16(skip) || !aligned16(output) || !aligned16(beta) || !aligned16(gamma)
+        || (bias && !aligned16(bias)))
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "SkipLayerNormDQQ: tensors must be 16-byte aligned");
+    }
+    constexpr int R = 4;
+    int64_t const rows = n / ld;
+    dim3 const grid((unsigned) ceil_div<int64_t>(ceil_div<int64_t>(rows, R), kWavesPerBlock));
+    auto const* b = reinterpret_cast<f16 const*>(beta);
+    auto const* g = reinterpret_cast<f16 const*>(gamma);
+    auto const* bs = reinterpret_cast<f16 const*>(bias);
+    if (bias)
+    {
+        hipLaunchKernelGGL((skipln_dqq_kernel<R, true>), grid, dim3(kBlock), 0, as_stream(stream), ld, rows, input,
+            skip, b, g, bs, output, dqScaleIn, dqScaleSkip, qScale);
+    }
+    else
+    {
+        hipLaunchKernelGGL((skipln_dqq_kernel<R, false>), grid, dim3(kBlock), 0, as_stream(stream), ld, rows, input,
+            skip, b, g, bs, output, dqScaleIn, dqScaleSkip, qScale);
+    }
+    return check_launch("skipln_dqq_kernel");
+}
+
+extern "C" int trtamd_skipln_interleaved_small_hface(trtamd_stream_t stream, int32_t ld, int32_t total,
+    int8_t const* input, int8_t const* skip, trtamd_half_t const* beta, trtamd_half_t const* gamma, int8_t* output,
+    float dqScaleIn, float dqScaleSkip, float qScale)
+{
+    return skipln_interleaved(as_stream(stream), false, false, ld, total, input, skip,
+        reinterpret_cast<f16 const*>(beta), reinterpret_cast<f16 const*>(gamma), output, nullptr, dqScaleIn,
+        dqScaleSkip, qScale, 0.f);
+}
+
+extern "C" int trtamd_skipln_interleaved_large_hface(trtamd_stream_t stream, int32_t ld, int32_t total,
+    int8_t const* input, int8_t const* skip, trtamd_half_t const* beta, trtamd_half_t const* gamma, int8_t* output,
+    float dqScaleIn, float dqScaleSkip, float qScale)
+{
+    return skipln_interleaved(as_stream(stream), true, false, ld, total, input, skip,
+        reinterpret_cast<f16 const*>(beta), reinterpret_cast<f16 const*>(gamma), output, nullptr, dqScaleIn,
+        dqScaleSkip, qScale, 0.f);
+}
+
+extern "C" int trtamd_skipln_interleaved_small_mtron(trtamd_stream_t stream, int32_t ld, int32_t total,
+    int8_t const* input, int8_t const* skip, trtamd_half_t const* beta, trtamd_half_t const* gamma, int8_t* output,
+    int8_t* preln, float dqScaleIn, float dqScaleSkip, float qScale, float qSkipScale)
+{
+    return skipln_interleaved(as_stream(stream), false, true, ld, total, input, skip,
+        reinterpret_cast<f16 const*>(beta), reinterpret_cast<f16 const*>(gamma), output, preln, dqScaleIn, dqScaleSkip,
+        qScale, qSkipScale);
+}
+
+extern "C" int trtamd_skipln_interleaved_large_mtron(trtamd_stream_t stream, int32_t ld, int32_t total,
+    int8_t const* input, int8_t const* skip, trtamd_half_t const* beta, trtamd_half_t const* gamma, int8_t* output,
+    int8_t* preln, float dqScaleIn, float dqScaleSkip, float qScale, float qSkipScale)
+{
+    return skipln_interleaved(as_stream(stream), true, true, ld, total, input, skip,
+        reinterpret_cast<f16 const*>(beta), reinterpret_cast<f16 const*>(gamma), output, preln, dqScaleIn, dqScaleSkip,
+        qScale, qSkipScale);
+}
