@@ -103,18 +103,29 @@ def test_fmha_int8_packed(api, B, N, S, rule, interleaved):
     got = host(d_out)
     got = oracle.deinterleave(got, T, N * D) if interleaved else got.reshape(T, N * D)
     g_a1, g_p8 = host(d_a1), host(d_p8)
-    maxl = int(lens.max())
+    ref = ref.reshape(T, N, D)
+    got3 = got.reshape(T, N, D)
+    n_p8 = n_off = 0
     for b in range(B):
         L = int(lens[b])
+        if L == 0:
+            continue
         assert np.array_equal(g_a1[b, :, :L, :L], a1[b, :, :L, :L]), "first-GEMM accumulators must be bit-exact"
-        assert_int8_close(g_p8[b, :, :L, :L], p8[b, :, :L, :L], what="quantised probabilities", max_frac_off=0.02)
+        dp = g_p8[b, :, :L, :L].astype(np.int32) - p8[b, :, :L, :L]
+        assert np.abs(dp).max() <= 1, "quantised probabilities differ by more than 1 LSB"
+        n_p8 += dp.size
+        n_off += int((dp != 0).sum())
         # exact second GEMM from the kernel's own p8
         v = qkv[cu[b]:cu[b + 1]].reshape(L, N, 3, D)[:, :, 2, :].astype(np.int64)      # [L,N,D]
         acc2 = np.einsum("nqk,knd->qnd", g_p8[b, :, :L, :L].astype(np.int64), v)        # [L,N,D]
-        want = np.clip(np.rint(acc2.astype(np.float32) * s2), -128, 127).astype(np.int8).reshape(L, N * D)
-        assert np.array_equal(got[cu[b]:cu[b + 1]], want), "second GEMM / requantisation must be exact"
-    assert maxl <= S
-    assert_int8_close(got, ref, what="context vs oracle", max_frac_off=0.05)
+        want = np.clip(np.rint(acc2.astype(np.float32) * s2), -128, 127).astype(np.int8)
+        assert np.array_equal(got3[cu[b]:cu[b + 1]], want), "second GEMM / requantisation must be exact"
+        # (query, head) rows whose probabilities agree with the oracle agree with it bit for bit;
+        # a probability that rounds the other way (exp differs in the last ulp) moves 64 outputs
+        # by up to |v| * scale_bmm2, which the exact check above already covers.
+        same = (dp == 0).all(axis=2).T                                                  # [L(q), N]
+        assert np.array_equal(got3[cu[b]:cu[b + 1]][same], ref[cu[b]:cu[b + 1]][same])
+    assert n_off <= max(2, 1e-5 * n_p8), f"{n_off} of {n_p8} probabilities differ from the oracle"
 
 
 @pytest.mark.parametrize("S,B,N", [(128, 3, 2), (384, 2, 3), (64, 4, 1), (96, 2, 2)])
