@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the BERT-large INT8 plugin path on one MI355X.
+
+One "step" = one encoder layer's plugin work over the whole batch, inputs resident in HBM:
+  CustomQKVToContextPluginDynamic v6 kernel (INT8, 32-interleaved, cu_seqlens)  ->
+  CustomSkipLayerNormPluginDynamic v7 kernel (INT8, 32-interleaved)
+on B=64 sequences, max length 384, lengths uniform in [192,384], 16 heads x 64 (hidden 1024).
+
+Prints ONE JSON line (see --help for flags): whole-job sequences/s, the roofline record of the
+dominant kernel (fused attention vs the dense INT8 MFMA peak), the other kernel's HBM roofline,
+and the CPU baseline (the C oracle timed on this host's cores on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "BERT-large INT8 S=384 seq/s on 1 GPU; % HBM peak (LN) & % INT8 MFMA peak (MHA)"
+PEAK_INT8_OPS = 5.0e15   # dense INT8 MFMA, op/s
+PEAK_HBM = 8.0e12        # B/s
+
+
+def f32_bits(x) -> int:
+    return int(np.float32(x).view(np.uint32))
+
+
+def build_inputs(B, S, seed):
+    import torch
+    from tensorrt_amd import workloads
+    wl = workloads.int8_layer(B, S, N=16, seed=seed)
+    T, E = wl.T, wl.E
+    d = {}
+    d["qkv"] = torch.from_numpy(workloads.interleave32(wl.qkv_tc)).cuda()
+    d["skip"] = torch.from_numpy(workloads.interleave32(wl.skip_tc)).cuda()
+    d["cu"] = torch.from_numpy(wl.cu).cuda()
+    d["gamma"] = torch.from_numpy(wl.gamma).cuda()
+    d["beta"] = torch.from_numpy(wl.beta).cuda()
+    d["ctx"] = torch.zeros(T * E, dtype=torch.int8, device="cuda")
+    d["out"] = torch.zeros(T * E, dtype=torch.int8, device="cuda")
+    # context scale = amax of the float attention of the dequantised tensor / 127, measured on the
+    # first sequences (set-up only; torch is not on the timed path)
+    x = torch.from_numpy(wl.qkv_tc[: int(wl.cu[2])].astype(np.float32) * float(wl.s_qkv)).cuda()
+    amax = 0.0
+    for b in range(2):
+        lo, hi = int(wl.cu[b]), int(wl.cu[b + 1])
+        q, k, v = (x[lo:hi, i * E:(i + 1) * E].reshape(hi - lo, wl.N, 64).transpose(0, 1) for i in range(3))
+        o = torch.softmax(q @ k.transpose(1, 2) / 8.0, -1) @ v
+        amax = max(amax, float(o.abs().max()))
+    s_ctx = np.float32(amax / 127.0)
+    # LayerNorm output scale: |gamma|max * ~4.5 sigma + |beta|max covers the normalised values
+    s_out = np.float32((float(np.abs(wl.gamma.astype(np.float32)).max()) * 4.5 + 0.5) / 127.0)
+    return wl, d, s_ctx, s_out
+
+
+def cpu_baseline(wl, s_ctx, s_out, budget_s=20.0):
+    """The C oracle (scalar restatement, OpenMP over sequences) on a bounded sample of the batch."""
+    import oracle
+    cores = len(os.sched_getaffinity(0))
+    threads = min(cores, 16)
+    os.environ["OMP_NUM_THREADS"] = str(threads)
+    nseq = min(wl.B, threads)
+    cu = wl.cu[: nseq + 1].copy()
+    T, E, N = int(cu[-1]), wl.E, wl.N
+    # oracle layout: [T, N, 3, d]
+    qkv = np.ascontiguousarray(wl.qkv_tc[:T].reshape(T, 3, N, 64).transpose(0, 2, 1, 3)).reshape(T, 3 * E)
+    s1 = np.float32(wl.s_qkv * wl.s_qkv * np.float32(0.125))
+    s2 = np.float32(wl.dq_probs * wl.s_qkv / s_ctx)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        ctx = oracle.mha_fused_i8_packed(qkv, cu, N, 64, s1, np.float32(127.0), s2)
+        st, _, _ = oracle.skipln_interleaved(0, oracle.interleave(ctx), oracle.interleave(wl.skip_tc[:T]), wl.beta,
+                                             wl.gamma, E, T, s_ctx, wl.s_skip, np.float32(1.0 / s_out), force=1)
+        assert st == 0
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s / 2 or reps >= 3:
+            break
+    return {"value": round(nseq * reps / el, 3), "unit": "sequences/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} pass(es) over the first {nseq} of {wl.B} sequences ({T} tokens): C oracle "
+                      f"orc_mha_fused_i8 + orc_skipln_interleaved, OpenMP over sequences, {el:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--seqlen", type=int, default=384)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every sequence, head and LayerNorm row "
+              "is independent; shard the batch). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from tensorrt_amd import capi
+    api = capi.api()   # raises if the HIP library is missing: there is no fallback
+
+    wl, d, s_ctx, s_out = build_inputs(args.batch, args.seqlen, args.seed)
+    T, E, N = wl.T, wl.E, wl.N
+    p = capi.FmhaParams()
+    p.qkv_ptr, p.o_ptr, p.cu_seqlens = d["qkv"].data_ptr(), d["ctx"].data_ptr(), d["cu"].data_ptr()
+    p.qkv_stride_in_bytes = p.o_stride_in_bytes = T
+    p.b, p.h, p.s, p.d = wl.B, N, wl.S, 64
+    p.scale_bmm1 = f32_bits(wl.s_qkv * wl.s_qkv * np.float32(0.125))
+    p.scale_softmax = f32_bits(1.0 / wl.dq_probs)
+    p.scale_bmm2 = f32_bits(wl.dq_probs * wl.s_qkv / s_ctx)
+    p.interleaved, p.use_int8_scale_max = 1, 1
+    stream = torch.cuda.current_stream().cuda_stream
+    q_out = np.float32(1.0 / s_out)
+
+    def mha():
+        api.check(api.fused_mha_run(stream, 2, C.byref(p)))
+
+    def skipln():
+        api.check(api.skipln_interleaved_large_hface(stream, E, T, d["ctx"].data_ptr(), d["skip"].data_ptr(),
+                                                      d["beta"].data_ptr(), d["gamma"].data_ptr(), d["out"].data_ptr(),
+                                                      s_ctx, wl.s_skip, q_out))
+
+    for _ in range(args.warmup):
+        mha()
+        skipln()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev[i][0].record()
+        mha()
+        ev[i][1].record()
+        skipln()
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / args.steps
+    t_mha = float(np.mean([e[0].elapsed_time(e[1]) for e in ev])) * 1e-3
+    t_ln = float(np.mean([e[1].elapsed_time(e[2]) for e in ev])) * 1e-3
+
+    mha_ops = wl.mha_ops()
+    ln_bytes = wl.skipln_bytes(1)
+    out = {
+        "metric": METRIC,
+        "value": round(wl.B / (ms_step * 1e-3), 1),
+        "unit": "sequences/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {
+            "workload": "BERT-large INT8 layer plugin path (configs[3]): QKV-to-context INT8 v6 kernel "
+                        "(32-interleaved, cu_seqlens) + SkipLayerNorm INT8 v7 kernel; the GEMMs between plugins are "
+                        "not part of the step",
+            "batch": wl.B, "max_seq_len": wl.S, "heads": N, "head_size": 64, "hidden": E, "tokens": T,
+            "lengths": f"uniform[{wl.S // 2},{wl.S}] seed {args.seed}",
+        },
+        "roofline": {
+            "kernel": "fmha_i8_kernel (interleaved)",
+            "bound": "mfma",
+            "achieved": round(mha_ops / t_mha / 1e12, 2),
+            "peak": PEAK_INT8_OPS / 1e12,
+            "unit": "TOP/s",
+            "frac": round(mha_ops / t_mha / PEAK_INT8_OPS, 4),
+            "traffic": None,
+            "avg_launch_us": round(t_mha * 1e6, 2),
+            "algorithmic_ops_per_launch": mha_ops,
+            "hbm_frac": round(wl.mha_bytes() / t_mha / PEAK_HBM, 4),
+        },
+        "roofline_skipln": {
+            "kernel": "skipln_interleaved_kernel<32,false>",
+            "bound": "hbm",
+            "achieved": round(ln_bytes / t_ln / 1e9, 1),
+            "peak": PEAK_HBM / 1e9,
+            "unit": "GB/s",
+            "frac": round(ln_bytes / t_ln / PEAK_HBM, 4),
+            "traffic": None,
+            "avg_launch_us": round(t_ln * 1e6, 2),
+            "algorithmic_bytes_per_launch": ln_bytes,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl, s_ctx, s_out)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

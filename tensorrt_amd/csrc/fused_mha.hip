@@ -4,24 +4,28 @@
 // the reference loads from cubins (plugin/bertQKVToContextPlugin/fused_multihead_attention*/):
 // one launch computes softmax(Q K^T * scale) V for every (sequence, head).
 //
-// Work split: a workgroup of 4 wavefronts owns 64 query rows of one (sequence, head); each wave
-// owns 16 of them and never talks to the others after the K/V tiles are staged.
-//   1. K is staged in LDS row-major (rows padded by 16 bytes so 16-byte reads of consecutive
-//      keys fall in different banks), V is staged transposed, [d][key], with the keys of each
-//      64-key block permuted into the order in which the MFMA accumulator of step 2 holds them.
-//   2. S^T = K Q^T with v_mfma_i32_16x16x64_i8 (v_mfma_f32_16x16x32_f16 for FP16): the
-//      accumulator layout gives every lane 4 keys x 1 query per 16-key tile, which is exactly
-//      the B-operand layout of step 4, so probabilities never leave registers.
-//   3. Row softmax over the whole row (<= 512 keys) held in registers: max/sum need only two
+// Work split: a workgroup stages K and V of one (sequence, head) in LDS once (both row-major, rows
+// padded by 16 bytes so 16-byte reads of consecutive keys fall in different banks) and its
+// wavefronts then walk the 16-row query tiles of that head round-robin; `qSplit` workgroups share
+// one head when the batch is too small to fill the chip otherwise.  Per query tile a wave
+//   1. computes S^T = K Q^T with v_mfma_i32_16x16x64_i8 (v_mfma_f32_16x16x32_f16 for FP16): the
+//      accumulator layout gives every lane 4 keys x 1 query per 16-key tile, which is exactly the
+//      B-operand layout of step 3, so probabilities never leave registers;
+//   2. does the row softmax over the whole row (<= 512 keys) in registers: max/sum need only two
 //      cross-lane steps (the 4 lane groups that share a query).  INT8 accumulators are seeded
 //      with the bit pattern of 1.5*2^23 so the integer result reads directly as a binary32
 //      number (no int->float conversion); probabilities are quantised with one fused
-//      multiply-add against the same constant (round-to-nearest-even lands in the low byte).
-//   4. O^T = V^T P^T with the same MFMA, requantised (INT8) or normalised (FP16) on store.
+//      multiply-add against the same constant (round-to-nearest-even lands in the low byte);
+//   3. computes O^T = V^T P^T with the same MFMA; the V^T operand (16 keys of one head-dim per
+//      lane) is produced from row-major V by the LDS transpose reads ds_read_b64_tr_b8 /
+//      ds_read_b64_tr_b16, so V is never transposed in memory;
+//   4. requantises (INT8) or normalises (FP16) on store.
 // Queries beyond the sequence length are neither computed nor written.
 #include "device_utils.hpp"
 #include "host_utils.hpp"
 
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -32,13 +36,16 @@ namespace
 {
 
 constexpr int kQPerWave = 16;
-constexpr int kWavesI8 = 4;  // 64 query rows per workgroup
-constexpr int kWavesF16 = 8; // 128 query rows per workgroup: FP16 K/V tiles take twice the LDS
+constexpr int kWavesI8 = 4;
+constexpr int kWavesF16 = 8; // FP16 K/V take twice the LDS, so one (larger) workgroup per CU
 constexpr int kHeadSize = 64;
 constexpr int kMagicBits = 0x4B400000;         // bit pattern of 12582912.f = 1.5 * 2^23
 constexpr float kMagic = 12582912.f;
-constexpr int kMaskedBits = 0x4B000000;        // below every reachable biased accumulator
 constexpr float kLog2e = 1.4426950408889634f;
+
+typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 
 struct FmhaArgs
 {
@@ -52,7 +59,7 @@ struct FmhaArgs
     int64_t seqStrideOut;
     int64_t maskStrideWords;
     int32_t B, N, S;
-    int32_t qTiles;              // ceil(S / query rows per workgroup)
+    int32_t qSplit;              // workgroups per (sequence, head)
     int32_t total;               // interleaved: total token count
     int32_t warpsM, warpsN;      // geometry of the packed mask
     float c;                     // scale_bmm1 * log2(e)
@@ -66,36 +73,43 @@ struct FmhaArgs
 template <int ESIZE>
 struct Lds
 {
-    // K rows of 64 elements padded by 16 bytes; V^T rows of (keys + pad) elements
-    static constexpr int kKRow = kHeadSize * ESIZE + 16;
-    static __host__ __device__ constexpr int vtRow(int kt)
+    // K and V rows of 64 elements, unpadded; the 16-byte chunks of a row are XOR-swizzled with
+    // the row index (see swz) so that the 8 consecutive rows a 16-lane group reads fall in
+    // different banks
+    static constexpr int kRow = kHeadSize * ESIZE;
+    static __host__ __device__ constexpr int matBytes(int kt)
     {
-        return kt * 64 * ESIZE + 16;
-    }
-    static __host__ __device__ constexpr int kBytes(int kt)
-    {
-        return kt * 64 * kKRow;
+        return kt * 64 * kRow;
     }
     static __host__ __device__ constexpr int total(int kt)
     {
-        return kBytes(kt) + kHeadSize * vtRow(kt) + 16 * 4;
+        return 2 * matBytes(kt) + 16 * 4;
     }
 };
 
-// Position, inside its 64-key block, at which key kk is stored in a V^T row.  The accumulator of
-// S^T gives lane group g the keys 16u + 4g + j (u = 16-key tile, j = 0..3) and the P^T operand is
-// built from it without moving data, so V^T must present keys in that order:
-//   INT8 (one MFMA per 64 keys, 16 slots per lane group): slot 4u + j   -> position 16g + 4u + j
-//   FP16 (one MFMA per 32 keys,  8 slots per lane group): slot 4(u&1)+j -> position 32(u/2) + 8g + 4(u&1) + j
+// LDS row, inside its 64-key block, at which V's key kk is stored.  The accumulator of S^T gives
+// lane group g the keys 16u + 4g + j (u = 16-key tile, j = 0..3) and the P^T operand is built
+// from it without moving data.  One INT8 transpose read returns 8 keys to each lane group, which
+// must be 8 consecutive LDS rows: tiles (2h, 2h+1), keys 4g..4g+3 of each -> rows 32h + 8g + 4(u&1) + j.
+// The FP16 transpose read returns 4 keys, already consecutive (16u + 4g + j): natural order.
 template <int ESIZE>
-__device__ inline int vt_pos(int kk)
+__device__ inline int v_row(int kk)
 {
     int const u = kk >> 4, g = (kk >> 2) & 3, j = kk & 3;
-    return ESIZE == 1 ? 16 * g + 4 * u + j : 32 * (u >> 1) + 8 * g + 4 * (u & 1) + j;
+    return ESIZE == 1 ? 32 * (u >> 1) + 8 * g + 4 * (u & 1) + j : kk;
 }
 
-// Byte address of the 16-byte chunk `chunk` (16*ESIZE... elements) of matrix `mat` (0 Q, 1 K, 2 V)
-// for head n, token `tok` of the sequence described by (base, tokStride).
+// Position of 16-byte chunk `chunk` inside LDS row `row`.  Rows are 64 (INT8) or 128 (FP16) bytes;
+// consecutive rows advance by a quarter / a half of the 256-byte bank window, so rows 2 (INT8) or
+// 1 (FP16) apart in the sense below would collide without the swizzle.
+template <int ESIZE>
+__device__ inline int swz(int row, int chunk)
+{
+    return ESIZE == 1 ? (chunk ^ ((row >> 1) & 3)) : (chunk ^ (row & 7));
+}
+
+// Byte address of the 16-byte chunk `chunk` of matrix `mat` (0 Q, 1 K, 2 V) for head n, token
+// `tok` of the sequence described by (seqBase, firstTok).
 template <int ESIZE, bool INTERLEAVED>
 __device__ inline int64_t qkv_chunk_offset(
     FmhaArgs const& a, int64_t seqBase, int64_t firstTok, int tok, int n, int mat, int chunk)
@@ -123,6 +137,7 @@ __device__ inline void build_key_mask(FmhaArgs const& a, int b, int nk, uint32_t
         }
         else
         {
+            // bit layout of fillSBSMaskKernel (plugin/embLayerNormPlugin/embLayerNormKernel.cu:41-85)
             uint32_t const* pm = a.packedMask + (int64_t) b * a.maskStrideWords;
             for (int i = 0; i < 32; ++i)
             {
@@ -144,66 +159,78 @@ __device__ inline void build_key_mask(FmhaArgs const& a, int b, int nk, uint32_t
     }
 }
 
-// Stage K (row-major, padded) and V (transposed, permuted) of one (sequence, head) into LDS.
-// Rows at or beyond nk are zero.  ESIZE = bytes per element (1 INT8, 2 FP16).
+// Stage K and V of one (sequence, head) into LDS, 16 bytes per lane per access.  Rows at or
+// beyond nk are zero, and so are the K rows of masked keys: a masked key's score is then exactly
+// the accumulator's seed, which the caller sets to -infinity (see mask_seed).  ESIZE = bytes per
+// element (1 INT8, 2 FP16).  sMask must be complete (barrier) before the call.
 template <int ESIZE, int KT, bool INTERLEAVED, int WAVES>
-__device__ inline void stage_kv(
-    FmhaArgs const& a, int64_t seqBase, int64_t firstTok, int n, int nk, int nkb, uint8_t* sK, uint8_t* sVT)
+__device__ inline void stage_kv(FmhaArgs const& a, int64_t seqBase, int64_t firstTok, int n, int nk, int nkb,
+    uint32_t const* sMask, uint8_t* sK, uint8_t* sV)
 {
     constexpr int kChunks = kHeadSize * ESIZE / 16;     // 16-byte chunks per head row: 4 or 8
     constexpr int kRowsPerPass = WAVES * kWaveSize / kChunks;
     constexpr int kPasses = 64 / kRowsPerPass;          // passes per 64-key block
-    constexpr int kVtRow = Lds<ESIZE>::vtRow(KT);
+    constexpr int kRow = Lds<ESIZE>::kRow;
     uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
     int const chunk = threadIdx.x % kChunks;
     int const rowInPass = threadIdx.x / kChunks;
+    // every global load of the workgroup is issued before the first LDS write, so the loads of
+    // all key blocks are in flight together
+    u32x4 kv[KT][kPasses], vv[KT][kPasses];
+#pragma unroll
+    for (int kb = 0; kb < KT; ++kb)
+    {
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p)
+        {
+            int const key = kb * 64 + p * kRowsPerPass + rowInPass;
+            kv[kb][p] = u32x4{0, 0, 0, 0};
+            vv[kb][p] = u32x4{0, 0, 0, 0};
+            if (key < nk)
+            {
+                vv[kb][p] = *reinterpret_cast<u32x4 const*>(
+                    src + qkv_chunk_offset<ESIZE, INTERLEAVED>(a, seqBase, firstTok, key, n, 2, chunk));
+                if ((sMask[key >> 5] >> (key & 31)) & 1u)
+                {
+                    kv[kb][p] = *reinterpret_cast<u32x4 const*>(
+                        src + qkv_chunk_offset<ESIZE, INTERLEAVED>(a, seqBase, firstTok, key, n, 1, chunk));
+                }
+            }
+        }
+    }
 #pragma unroll
     for (int kb = 0; kb < KT; ++kb)
     {
         if (kb < nkb)
         {
-            u32x4 kv[kPasses], vv[kPasses];
-#pragma unroll
-            for (int p = 0; p < kPasses; ++p)
-            {
-                int const key = kb * 64 + p * kRowsPerPass + rowInPass;
-                kv[p] = u32x4{0, 0, 0, 0};
-                vv[p] = u32x4{0, 0, 0, 0};
-                if (key < nk)
-                {
-                    kv[p] = *reinterpret_cast<u32x4 const*>(
-                        src + qkv_chunk_offset<ESIZE, INTERLEAVED>(a, seqBase, firstTok, key, n, 1, chunk));
-                    vv[p] = *reinterpret_cast<u32x4 const*>(
-                        src + qkv_chunk_offset<ESIZE, INTERLEAVED>(a, seqBase, firstTok, key, n, 2, chunk));
-                }
-            }
 #pragma unroll
             for (int p = 0; p < kPasses; ++p)
             {
                 int const kk = p * kRowsPerPass + rowInPass;
-                int const key = kb * 64 + kk;
-                *reinterpret_cast<u32x4*>(sK + key * Lds<ESIZE>::kKRow + chunk * 16) = kv[p];
-                int const col = (kb * 64 + vt_pos<ESIZE>(kk)) * ESIZE;
-                if (ESIZE == 1)
-                {
-#pragma unroll
-                    for (int x = 0; x < 16; ++x)
-                    {
-                        sVT[(chunk * 16 + x) * kVtRow + col] = (uint8_t) (vv[p][x >> 2] >> (8 * (x & 3)));
-                    }
-                }
-                else
-                {
-#pragma unroll
-                    for (int x = 0; x < 8; ++x)
-                    {
-                        *reinterpret_cast<uint16_t*>(sVT + (chunk * 8 + x) * kVtRow + col)
-                            = (uint16_t) (vv[p][x >> 1] >> (16 * (x & 1)));
-                    }
-                }
+                int const kr = kb * 64 + kk;
+                int const vr = kb * 64 + v_row<ESIZE>(kk);
+                *reinterpret_cast<u32x4*>(sK + kr * kRow + swz<ESIZE>(kr, chunk) * 16) = kv[kb][p];
+                *reinterpret_cast<u32x4*>(sV + vr * kRow + swz<ESIZE>(vr, chunk) * 16) = vv[kb][p];
             }
         }
     }
+}
+
+// Accumulator seed of the four keys 16u + 4g + j of a 16-key tile: `valid` for keys that take
+// part, the bit pattern of -infinity for masked ones (their K rows are zero, so the seed is their
+// score): the integer/float row maximum ignores it and 2^(-inf) = 0 removes it from the softmax
+// without any per-score instruction.
+constexpr int kNegInfBits = (int) 0xFF800000u;
+__device__ inline i32x4 mask_seed(uint32_t w0, uint32_t w1, int u, int g, int valid)
+{
+    uint32_t const bits = ((u < 2 ? w0 : w1) >> ((u & 1) * 16 + g * 4)) & 0xfu;
+    i32x4 seed;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        seed[j] = (bits >> j) & 1u ? valid : kNegInfBits;
+    }
+    return seed;
 }
 
 struct SeqInfo
@@ -236,242 +263,332 @@ __device__ inline SeqInfo seq_info(FmhaArgs const& a, int b, int capacity)
     return s;
 }
 
+// Which sequence a workgroup serves.  Workgroups are dispatched in index order, so serving the
+// longest sequences first (cost grows with the square of the length) lets the short ones fill the
+// tail of the launch.  `rank` is the position in that order; every workgroup ranks the (at most
+// kMaxRanked) sequence lengths itself with a counting sort in LDS: no state outside the launch.
+constexpr int kMaxRanked = 1024;
+template <int THREADS>
+__device__ inline int pick_sequence(FmhaArgs const& a, int rank, int* sLens /* [kMaxRanked + 1] */)
+{
+    if (a.cuSeqlens == nullptr || a.B > kMaxRanked || a.B == 1)
+    {
+        return rank; // fixed layout (equal lengths) or too many sequences: natural order
+    }
+    for (int t = threadIdx.x; t < a.B; t += THREADS)
+    {
+        sLens[t] = a.cuSeqlens[t + 1] - a.cuSeqlens[t];
+    }
+    if (threadIdx.x == 0)
+    {
+        sLens[kMaxRanked] = rank;
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < a.B; t += THREADS)
+    {
+        int const mine = sLens[t];
+        int before = 0; // sequences served before t: longer ones, ties by index
+        for (int o = 0; o < a.B; ++o)
+        {
+            int const other = sLens[o];
+            before += (other > mine || (other == mine && o < t)) ? 1 : 0;
+        }
+        if (before == rank)
+        {
+            sLens[kMaxRanked] = t;
+        }
+    }
+    __syncthreads();
+    return sLens[kMaxRanked];
+}
+
 // ------------------------------------------------------------------------------------------
 // INT8
 // ------------------------------------------------------------------------------------------
 template <int KT, bool INTERLEAVED, bool DEBUG>
-__global__ __launch_bounds__(kWavesI8* kWaveSize) void fmha_i8_kernel(FmhaArgs const a)
+__global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_per_eu(KT <= 6 ? 3 : 2))) void fmha_i8_kernel(FmhaArgs const a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* sK = smem;
-    uint8_t* sVT = smem + Lds<1>::kBytes(KT);
-    uint32_t* sMask = reinterpret_cast<uint32_t*>(sVT + kHeadSize * Lds<1>::vtRow(KT));
-    constexpr int kVtRow = Lds<1>::vtRow(KT);
-    constexpr int kKRow = Lds<1>::kKRow;
+    uint8_t* sV = smem + Lds<1>::matBytes(KT);
+    uint32_t* sMask = reinterpret_cast<uint32_t*>(sV + Lds<1>::matBytes(KT));
+    constexpr int kRow = Lds<1>::kRow;
 
-    uint32_t const bid = xcd_remap(blockIdx.x, gridDim.x);
-    int const qt = bid % a.qTiles;
-    int const n = (bid / a.qTiles) % a.N;
-    int const b = bid / (a.qTiles * a.N);
+    __shared__ int sLens[kMaxRanked + 1];
+    // workgroup ids are dealt round-robin to the 8 XCDs: when a head is split over several
+    // workgroups, renumber so that they land on one XCD and share K/V in its L2
+    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
+    int const part = bid % a.qSplit;
+    int const n = (bid / a.qSplit) % a.N;
+    int const b = pick_sequence<kWavesI8 * kWaveSize>(a, bid / (a.qSplit * a.N), sLens);
     SeqInfo const sq = seq_info(a, b, KT * 64);
-    int const q0 = qt * (kWavesI8 * kQPerWave);
-    if (q0 >= sq.nq)
+    int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
+    if (part * kWavesI8 >= nqt)
     {
-        return;
+        return; // no query tile for this workgroup
     }
     int const nkb = (sq.nk + 63) >> 6;
+    int const ntile = (sq.nk + 15) >> 4; // 16-key tiles that hold at least one key
     build_key_mask(a, b, sq.nk, sMask);
-    stage_kv<1, KT, INTERLEAVED, kWavesI8>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sK, sVT);
+    __syncthreads();
+    stage_kv<1, KT, INTERLEAVED, kWavesI8>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sMask, sK, sV);
+    __syncthreads();
 
     int const lane = threadIdx.x & (kWaveSize - 1);
     int const wave = threadIdx.x >> 6;
     int const lq = lane & 15; // query (column of S^T / O^T)
     int const g = lane >> 4;  // lane group: 16-byte k-chunk of the operands, 4 rows of the accumulators
-    int const q = q0 + wave * kQPerWave + lq;
-    bool const qValid = q < sq.nq;
+    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
 
-    // Q^T operand: 16 bytes d = 16g .. 16g+15 of query q
-    i32x4 qreg = {0, 0, 0, 0};
-    if (qValid)
-    {
-        qreg = *reinterpret_cast<i32x4 const*>(static_cast<uint8_t const*>(a.qkv)
-            + qkv_chunk_offset<1, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, q, n, 0, g));
-    }
-    __syncthreads();
-    if (q0 + wave * kQPerWave >= sq.nq)
-    {
-        return; // this wave's 16 rows lie beyond the sequence (no barrier follows)
-    }
-
-    // ---- S^T = K Q^T, biased so that the int32 reads as binary32 12582912 + acc ------------
-    i32x4 acc[KT * 4];
-#pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
+    // Q^T operand of a tile: 16 bytes d = 16g .. 16g+15 of query 16*qt + lq (zero beyond the
+    // sequence).  The next tile's operand is requested while the current tile is computed.
+    auto load_q = [&](int qt) -> i32x4 {
+        int const qq = qt * kQPerWave + lq;
+        i32x4 v = {0, 0, 0, 0};
+        if (qq < sq.nq)
         {
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-            {
-                int const key = kb * 64 + u * 16 + lq;
-                i32x4 const kreg = *reinterpret_cast<i32x4 const*>(sK + key * kKRow + g * 16);
-                acc[kb * 4 + u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                    kreg, qreg, i32x4{kMagicBits, kMagicBits, kMagicBits, kMagicBits}, 0, 0, 0);
-            }
+            v = *reinterpret_cast<i32x4 const*>(
+                src + qkv_chunk_offset<1, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, g));
         }
-    }
-
-    if (DEBUG && a.dbgAcc1 && qValid)
+        return v;
+    };
+    int const qtStep = a.qSplit * kWavesI8;
+    i32x4 qnext = load_q(part * kWavesI8 + wave);
+    for (int qt = part * kWavesI8 + wave; qt < nqt; qt += qtStep)
     {
+        int const q = qt * kQPerWave + lq;
+        bool const qValid = q < sq.nq;
+        i32x4 const qreg = qnext;
+        qnext = load_q(qt + qtStep);
+
+        // ---- S^T = K Q^T, biased so that the int32 reads as binary32 12582912 + acc --------
+        i32x4 acc[KT * 4];
 #pragma unroll
         for (int kb = 0; kb < KT; ++kb)
         {
             if (kb < nkb)
             {
+                uint32_t const w0 = __builtin_amdgcn_readfirstlane(sMask[kb * 2]);
+                uint32_t const w1 = __builtin_amdgcn_readfirstlane(sMask[kb * 2 + 1]);
+                bool const full = (w0 & w1) == 0xffffffffu;
+#pragma unroll
                 for (int u = 0; u < 4; ++u)
                 {
-                    for (int j = 0; j < 4; ++j)
+                    if (kb * 4 + u >= ntile)
                     {
-                        int const key = kb * 64 + u * 16 + g * 4 + j;
-                        if (key < sq.nk)
+                        break; // tiles wholly beyond the sequence are never touched
+                    }
+                    int const key = kb * 64 + u * 16 + lq;
+                    i32x4 const kreg = *reinterpret_cast<i32x4 const*>(sK + key * kRow + swz<1>(key, g) * 16);
+                    i32x4 seed = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
+                    if (!full)
+                    {
+                        asm volatile("" ::: "memory"); // scalar branch, taken for the ragged last block only
+                        seed = mask_seed(w0, w1, u, g, kMagicBits);
+                    }
+                    acc[kb * 4 + u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kreg, qreg, seed, 0, 0, 0);
+                }
+            }
+        }
+
+        if (DEBUG && a.dbgAcc1 && qValid)
+        {
+#pragma unroll
+            for (int kb = 0; kb < KT; ++kb)
+            {
+                if (kb < nkb)
+                {
+                    for (int u = 0; u < 4; ++u)
+                    {
+                        for (int j = 0; j < 4; ++j)
                         {
-                            a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key] = acc[kb * 4 + u][j] - kMagicBits;
+                            int const key = kb * 64 + u * 16 + g * 4 + j;
+                            if (key < sq.nk)
+                            {
+                                a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
+                                    = acc[kb * 4 + u][j] - kMagicBits;
+                            }
                         }
                     }
                 }
             }
         }
-    }
 
-    // ---- mask + row max (on the biased integers: the bias is monotone) ---------------------
-    int mx = kMaskedBits;
+        // ---- row max on the biased integers (the bias is monotone; masked keys hold the
+        //      negative pattern of -infinity) ------------------------------------------------------
+        int mx = kNegInfBits;
 #pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
+        for (int kb = 0; kb < KT; ++kb)
         {
-            uint32_t const w0 = __builtin_amdgcn_readfirstlane(sMask[kb * 2]);
-            uint32_t const w1 = __builtin_amdgcn_readfirstlane(sMask[kb * 2 + 1]);
-            bool const full = (w0 & w1) == 0xffffffffu;
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
+            if (kb < nkb)
             {
-                if (!full)
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
                 {
-                    uint32_t const bits = ((u < 2 ? w0 : w1) >> ((u & 1) * 16 + g * 4)) & 0xfu;
+                    if (kb * 4 + u >= ntile)
+                    {
+                        break;
+                    }
+                    mx = max(mx, max(max(acc[kb * 4 + u][0], acc[kb * 4 + u][1]),
+                                     max(acc[kb * 4 + u][2], acc[kb * 4 + u][3])));
+                }
+            }
+        }
+        mx = max(mx, __shfl_xor(mx, 16, kWaveSize));
+        mx = max(mx, __shfl_xor(mx, 32, kWaveSize));
+
+        // ---- e = 2^((acc - max) * c), row sum; a fully masked row has max = -inf -> all e = 0 --
+        float const negK0 = mx == kNegInfBits ? 0.f : -__int_as_float(mx) * a.c;
+        float sum = 0.f;
+        // e overwrites the accumulators in place (as bit patterns) to keep one row in registers
+#pragma unroll
+        for (int kb = 0; kb < KT; ++kb)
+        {
+            if (kb < nkb)
+            {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                {
+                    if (kb * 4 + u >= ntile)
+                    {
+                        break;
+                    }
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                     {
-                        acc[kb * 4 + u][j] = (bits >> j) & 1u ? acc[kb * 4 + u][j] : kMaskedBits;
+                        float const ev
+                            = __builtin_amdgcn_exp2f(fmaf(__int_as_float(acc[kb * 4 + u][j]), a.c, negK0));
+                        acc[kb * 4 + u][j] = __float_as_int(ev);
+                        sum += ev;
                     }
                 }
-                mx = max(mx, max(max(acc[kb * 4 + u][0], acc[kb * 4 + u][1]),
-                                 max(acc[kb * 4 + u][2], acc[kb * 4 + u][3])));
             }
         }
-    }
-    mx = max(mx, __shfl_xor(mx, 16, kWaveSize));
-    mx = max(mx, __shfl_xor(mx, 32, kWaveSize));
-
-    // ---- e = 2^((acc - max) * c), row sum -----------------------------------------------------
-    float const negK0 = -__int_as_float(mx) * a.c;
-    float sum = 0.f;
-    float e[KT * 4][4];
-#pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
+        sum += __shfl_xor(sum, 16, kWaveSize);
+        sum += __shfl_xor(sum, 32, kWaveSize);
+        float const r = sum > 0.f ? a.scaleSoftmax / sum : 0.f;
+        // e * r <= scale_softmax: only a scale above 127 can leave the INT8 range; the row is then
+        // pre-clamped through e <= 127 / r (one extra op per score on that rare path only)
+        if (a.clampP)
         {
-            uint32_t const w0 = __builtin_amdgcn_readfirstlane(sMask[kb * 2]);
-            uint32_t const w1 = __builtin_amdgcn_readfirstlane(sMask[kb * 2 + 1]);
-            bool const full = (w0 & w1) == 0xffffffffu;
+            asm volatile("" ::: "memory"); // keep this a scalar branch: the clamp must not be speculated
+            float const emax = r > 0.f ? 127.f / r : 0.f;
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int kb = 0; kb < KT; ++kb)
             {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
+                if (kb < nkb)
                 {
-                    float v = __builtin_amdgcn_exp2f(fmaf(__int_as_float(acc[kb * 4 + u][j]), a.c, negK0));
-                    if (!full)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
                     {
-                        v = acc[kb * 4 + u][j] == kMaskedBits ? 0.f : v;
+                        if (kb * 4 + u >= ntile)
+                        {
+                            break;
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                        {
+                            acc[kb * 4 + u][j] = __float_as_int(fminf(__int_as_float(acc[kb * 4 + u][j]), emax));
+                        }
                     }
-                    e[kb * 4 + u][j] = v;
-                    sum += v;
                 }
             }
         }
-    }
-    sum += __shfl_xor(sum, 16, kWaveSize);
-    sum += __shfl_xor(sum, 32, kWaveSize);
-    float const r = sum > 0.f ? a.scaleSoftmax / sum : 0.f;
 
-    // ---- p8 = rne(e * r) packed four keys to a dword; O^T = V^T P^T ---------------------------
-    i32x4 oacc[4];
+        // ---- p8 = rne(e * r) packed four keys to a dword; O^T = V^T P^T -----------------------
+        i32x4 oacc[4];
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-    {
-        oacc[dt] = i32x4{0, 0, 0, 0};
-    }
-#pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
+        for (int dt = 0; dt < 4; ++dt)
         {
-            i32x4 preg;
+            oacc[dt] = i32x4{0, 0, 0, 0};
+        }
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+        for (int kb = 0; kb < KT; ++kb)
+        {
+            if (kb < nkb)
+            {
+                i32x4 preg = {0, 0, 0, 0};
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                {
+                    if (kb * 4 + u >= ntile)
+                    {
+                        break;
+                    }
+                    uint32_t yb[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        yb[j] = __float_as_uint(fmaf(__int_as_float(acc[kb * 4 + u][j]), r, kMagic));
+                    }
+                    uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+                    uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+                    preg[u] = (int) __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                }
+                if (DEBUG && a.dbgP8 && qValid)
+                {
+                    for (int u = 0; u < 4; ++u)
+                    {
+                        for (int j = 0; j < 4; ++j)
+                        {
+                            int const key = kb * 64 + u * 16 + g * 4 + j;
+                            if (key < sq.nk)
+                            {
+                                a.dbgP8[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
+                                    = (int8_t) ((uint32_t) preg[u] >> (8 * j));
+                            }
+                        }
+                    }
+                }
+                // V^T operand for head dims 16dt .. 16dt+15: lane r of a group addresses LDS row
+                // (8 keys per read: r/2) at byte 16dt + 8(r%2); the transpose read hands lane i
+                // the 8 keys of head dim 16dt + i.
+                int const vrow = kb * 64 + 8 * g + (lq >> 1);
+                uint8_t const* vbase = sV + vrow * kRow + 8 * (lq & 1);
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+                {
+                    // rows vrow and vrow + 32 share (row >> 1) & 3, hence the swizzled chunk
+                    int const sc = swz<1>(vrow, dt) * 16;
+                    i32x2 const v0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + sc));
+                    i32x2 const v1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + 32 * kRow + sc));
+                    i32x4 const vreg = {v0[0], v0[1], v1[0], v1[1]};
+                    oacc[dt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vreg, preg, oacc[dt], 0, 0, 0);
+                }
+            }
+        }
+
+        // ---- out8 = sat8(rne(acc2 * scale_bmm2)); lane holds d = 16dt + 4g .. +3 of query q --
+        if (qValid)
+        {
+            uint8_t* dst = static_cast<uint8_t*>(a.out);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
             {
                 uint32_t yb[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                 {
-                    float y = e[kb * 4 + u][j] * r;
-                    if (a.clampP)
-                    {
-                        y = fminf(y, 127.f);
-                    }
+                    float y = (float) oacc[dt][j] * a.scaleBmm2;
+                    y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
                     yb[j] = __float_as_uint(y + kMagic);
                 }
                 uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
                 uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-                preg[u] = (int) __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-            }
-            if (DEBUG && a.dbgP8 && qValid)
-            {
-                for (int u = 0; u < 4; ++u)
+                uint32_t const packed = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                int const d0 = dt * 16 + g * 4;
+                int64_t off;
+                if (INTERLEAVED)
                 {
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        int const key = kb * 64 + u * 16 + g * 4 + j;
-                        if (key < sq.nk)
-                        {
-                            a.dbgP8[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
-                                = (int8_t) ((uint32_t) preg[u] >> (8 * j));
-                        }
-                    }
+                    // [N][d/32][T][32]
+                    off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
                 }
+                else
+                {
+                    off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
+                }
+                *reinterpret_cast<uint32_t*>(dst + off) = packed;
             }
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-            {
-                i32x4 const vreg
-                    = *reinterpret_cast<i32x4 const*>(sVT + (dt * 16 + lq) * kVtRow + kb * 64 + g * 16);
-                oacc[dt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vreg, preg, oacc[dt], 0, 0, 0);
-            }
-        }
-    }
-
-    // ---- out8 = sat8(rne(acc2 * scale_bmm2)); lane holds d = 16dt + 4g .. +3 of query q ------
-    if (qValid)
-    {
-        uint8_t* dst = static_cast<uint8_t*>(a.out);
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-        {
-            uint32_t yb[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-            {
-                float y = (float) oacc[dt][j] * a.scaleBmm2;
-                y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
-                yb[j] = __float_as_uint(y + kMagic);
-            }
-            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
-            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-            uint32_t const packed = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-            int const d0 = dt * 16 + g * 4;
-            int64_t off;
-            if (INTERLEAVED)
-            {
-                // [N][d/32][T][32]
-                off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
-            }
-            else
-            {
-                off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
-            }
-            *reinterpret_cast<uint32_t*>(dst + off) = packed;
         }
     }
 }
@@ -484,211 +601,214 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* sK = smem;
-    uint8_t* sVT = smem + Lds<2>::kBytes(KT);
-    uint32_t* sMask = reinterpret_cast<uint32_t*>(sVT + kHeadSize * Lds<2>::vtRow(KT));
-    constexpr int kVtRow = Lds<2>::vtRow(KT);
-    constexpr int kKRow = Lds<2>::kKRow;
+    uint8_t* sV = smem + Lds<2>::matBytes(KT);
+    uint32_t* sMask = reinterpret_cast<uint32_t*>(sV + Lds<2>::matBytes(KT));
+    constexpr int kRow = Lds<2>::kRow;
 
-    uint32_t const bid = xcd_remap(blockIdx.x, gridDim.x);
-    int const qt = bid % a.qTiles;
-    int const n = (bid / a.qTiles) % a.N;
-    int const b = bid / (a.qTiles * a.N);
+    __shared__ int sLens[kMaxRanked + 1];
+    // workgroup ids are dealt round-robin to the 8 XCDs: when a head is split over several
+    // workgroups, renumber so that they land on one XCD and share K/V in its L2
+    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
+    int const part = bid % a.qSplit;
+    int const n = (bid / a.qSplit) % a.N;
+    int const b = pick_sequence<kWavesF16 * kWaveSize>(a, bid / (a.qSplit * a.N), sLens);
     SeqInfo const sq = seq_info(a, b, KT * 64);
-    int const q0 = qt * (kWavesF16 * kQPerWave);
-    if (q0 >= sq.nq)
+    int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
+    if (part * kWavesF16 >= nqt)
     {
         return;
     }
     int const nkb = (sq.nk + 63) >> 6;
     build_key_mask(a, b, sq.nk, sMask);
-    stage_kv<2, KT, false, kWavesF16>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sK, sVT);
+    __syncthreads();
+    stage_kv<2, KT, false, kWavesF16>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sMask, sK, sV);
+    __syncthreads();
 
     int const lane = threadIdx.x & (kWaveSize - 1);
     int const wave = threadIdx.x >> 6;
     int const lq = lane & 15;
     int const g = lane >> 4;
-    int const q = q0 + wave * kQPerWave + lq;
-    bool const qValid = q < sq.nq;
-
-    // Q^T operands: MFMA h covers d = 32h + 8g .. +7
-    f16x8 qreg[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-    {
-        u32x4 raw = {0, 0, 0, 0};
-        if (qValid)
-        {
-            raw = *reinterpret_cast<u32x4 const*>(static_cast<uint8_t const*>(a.qkv)
-                + qkv_chunk_offset<2, false>(a, sq.seqBaseIn, sq.firstTok, q, n, 0, h * 4 + g));
-        }
-        qreg[h] = __builtin_bit_cast(f16x8, raw);
-    }
-    __syncthreads();
-    if (q0 + wave * kQPerWave >= sq.nq)
-    {
-        return;
-    }
-
-    // ---- S^T = K Q^T (binary32 accumulation) ---------------------------------------------------
-    f32x4 acc[KT * 4];
-#pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
-        {
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-            {
-                int const key = kb * 64 + u * 16 + lq;
-                f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-                {
-                    f16x8 const kreg = *reinterpret_cast<f16x8 const*>(sK + key * kKRow + (h * 4 + g) * 16);
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg, qreg[h], s, 0, 0, 0);
-                }
-                acc[kb * 4 + u] = s;
-            }
-        }
-    }
-
-    if (DEBUG && a.dbgAcc1 && qValid)
-    {
-#pragma unroll
-        for (int kb = 0; kb < KT; ++kb)
-        {
-            if (kb < nkb)
-            {
-                for (int u = 0; u < 4; ++u)
-                {
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        int const key = kb * 64 + u * 16 + g * 4 + j;
-                        if (key < sq.nk)
-                        {
-                            a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
-                                = __float_as_int(acc[kb * 4 + u][j]);
-                        }
-                    }
-                }
-            }
-        }
-    }
-
-    // ---- mask + row max ------------------------------------------------------------------------
-    constexpr float kNegBig = -3.0e38f;
-    float mx = kNegBig;
-#pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
-        {
-            uint32_t const w0 = __builtin_amdgcn_readfirstlane(sMask[kb * 2]);
-            uint32_t const w1 = __builtin_amdgcn_readfirstlane(sMask[kb * 2 + 1]);
-            bool const full = (w0 & w1) == 0xffffffffu;
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-            {
-                if (!full)
-                {
-                    uint32_t const bits = ((u < 2 ? w0 : w1) >> ((u & 1) * 16 + g * 4)) & 0xfu;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        acc[kb * 4 + u][j] = (bits >> j) & 1u ? acc[kb * 4 + u][j] : kNegBig;
-                    }
-                }
-                mx = fmaxf(mx, fmaxf(fmaxf(acc[kb * 4 + u][0], acc[kb * 4 + u][1]),
-                                     fmaxf(acc[kb * 4 + u][2], acc[kb * 4 + u][3])));
-            }
-        }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, kWaveSize));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWaveSize));
-
-    // ---- p = 2^((s - max) * c) rounded to binary16; O^T = V^T P^T; the row sum is taken by the
-    //      matrix unit as well (a tile of ones), so numerator and denominator see the same
-    //      rounded probabilities -------------------------------------------------------------------
-    float const negK0 = -mx * a.c;
-    f32x4 oacc[4];
-    f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-    {
-        oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
+    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
     f16x8 ones;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
     {
         ones[i] = (f16) 1.f;
     }
-#pragma unroll
-    for (int kb = 0; kb < KT; ++kb)
-    {
-        if (kb < nkb)
+
+    // Q^T operands of a tile: MFMA h covers d = 32h + 8g .. +7 of query 16*qt + lq.  The next
+    // tile's operands are requested while the current tile is computed.
+    auto load_q = [&](int qt, int h) -> f16x8 {
+        int const qq = qt * kQPerWave + lq;
+        u32x4 raw = {0, 0, 0, 0};
+        if (qq < sq.nq)
         {
-            uint32_t const w0 = __builtin_amdgcn_readfirstlane(sMask[kb * 2]);
-            uint32_t const w1 = __builtin_amdgcn_readfirstlane(sMask[kb * 2 + 1]);
-            bool const full = (w0 & w1) == 0xffffffffu;
+            raw = *reinterpret_cast<u32x4 const*>(
+                src + qkv_chunk_offset<2, false>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, h * 4 + g));
+        }
+        return __builtin_bit_cast(f16x8, raw);
+    };
+    int const qtStep = a.qSplit * kWavesF16;
+    f16x8 qnext[2] = {load_q(part * kWavesF16 + wave, 0), load_q(part * kWavesF16 + wave, 1)};
+    for (int qt = part * kWavesF16 + wave; qt < nqt; qt += qtStep)
+    {
+        int const q = qt * kQPerWave + lq;
+        bool const qValid = q < sq.nq;
+        f16x8 const qreg[2] = {qnext[0], qnext[1]};
+        qnext[0] = load_q(qt + qtStep, 0);
+        qnext[1] = load_q(qt + qtStep, 1);
+
+        // ---- S^T = K Q^T (binary32 accumulation) -----------------------------------------------
+        f32x4 acc[KT * 4];
 #pragma unroll
-            for (int hb = 0; hb < 2; ++hb) // 32-key half of the block
+        for (int kb = 0; kb < KT; ++kb)
+        {
+            if (kb < nkb)
             {
-                f16x8 preg;
+                uint32_t const w0 = __builtin_amdgcn_readfirstlane(sMask[kb * 2]);
+                uint32_t const w1 = __builtin_amdgcn_readfirstlane(sMask[kb * 2 + 1]);
+                bool const full = (w0 & w1) == 0xffffffffu;
 #pragma unroll
-                for (int w = 0; w < 2; ++w)
+                for (int u = 0; u < 4; ++u)
                 {
-                    int const t = kb * 4 + hb * 2 + w;
-                    float p[4];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                    int const key = kb * 64 + u * 16 + lq;
+                    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+                    if (!full)
                     {
-                        float v = __builtin_amdgcn_exp2f(fmaf(acc[t][j], a.c, negK0));
-                        if (!full)
-                        {
-                            v = acc[t][j] == kNegBig ? 0.f : v;
-                        }
-                        p[j] = v;
+                        asm volatile("" ::: "memory"); // scalar branch, taken for the ragged last block only
+                        s = __builtin_bit_cast(f32x4, mask_seed(w0, w1, u, g, 0));
                     }
-                    f16x2 const p01 = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(p[0], p[1]));
-                    f16x2 const p23 = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(p[2], p[3]));
-                    preg[w * 4 + 0] = p01[0];
-                    preg[w * 4 + 1] = p01[1];
-                    preg[w * 4 + 2] = p23[0];
-                    preg[w * 4 + 3] = p23[1];
-                }
-                if (DEBUG && a.dbgP8)
-                {
-                    // not used for FP16
-                }
 #pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
-                {
-                    f16x8 const vreg = *reinterpret_cast<f16x8 const*>(
-                        sVT + (dt * 16 + lq) * kVtRow + ((kb * 64 + hb * 32) + g * 8) * 2);
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg, preg, oacc[dt], 0, 0, 0);
+                    for (int h = 0; h < 2; ++h)
+                    {
+                        f16x8 const kreg
+                            = *reinterpret_cast<f16x8 const*>(sK + key * kRow + swz<2>(key, h * 4 + g) * 16);
+                        s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg, qreg[h], s, 0, 0, 0);
+                    }
+                    acc[kb * 4 + u] = s;
                 }
-                sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, preg, sacc, 0, 0, 0);
             }
         }
-    }
 
-    if (qValid)
-    {
-        float const rinv = sacc[0] > 0.f ? 1.f / sacc[0] : 0.f;
-        uint8_t* dst = static_cast<uint8_t*>(a.out);
+        if (DEBUG && a.dbgAcc1 && qValid)
+        {
+#pragma unroll
+            for (int kb = 0; kb < KT; ++kb)
+            {
+                if (kb < nkb)
+                {
+                    for (int u = 0; u < 4; ++u)
+                    {
+                        for (int j = 0; j < 4; ++j)
+                        {
+                            int const key = kb * 64 + u * 16 + g * 4 + j;
+                            if (key < sq.nk)
+                            {
+                                a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
+                                    = __float_as_int(acc[kb * 4 + u][j]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+
+        // ---- row max (masked keys hold -infinity) ------------------------------------------------
+        float mx = -__builtin_inff();
+#pragma unroll
+        for (int kb = 0; kb < KT; ++kb)
+        {
+            if (kb < nkb)
+            {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                {
+                    mx = fmaxf(mx, fmaxf(fmaxf(acc[kb * 4 + u][0], acc[kb * 4 + u][1]),
+                                         fmaxf(acc[kb * 4 + u][2], acc[kb * 4 + u][3])));
+                }
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, kWaveSize));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWaveSize));
+
+        // ---- p = 2^((s - max) * c) rounded to binary16; O^T = V^T P^T; the row sum is taken by
+        //      the matrix unit as well (a tile of ones), so numerator and denominator see the
+        //      same rounded probabilities ---------------------------------------------------------
+        float const negK0 = mx == -__builtin_inff() ? 0.f : -mx * a.c; // fully masked row: every p = 0
+        f32x4 oacc[4];
+        f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
         {
-            f16x4 y;
+            oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+        for (int kb = 0; kb < KT; ++kb)
+        {
+            if (kb < nkb)
             {
-                y[j] = (f16) (oacc[dt][j] * rinv);
+#pragma unroll
+                for (int hb = 0; hb < 2; ++hb) // 32-key half of the block
+                {
+                    f16x8 preg;
+#pragma unroll
+                    for (int w = 0; w < 2; ++w)
+                    {
+                        int const t = kb * 4 + hb * 2 + w;
+                        float p[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                        {
+                            p[j] = __builtin_amdgcn_exp2f(fmaf(acc[t][j], a.c, negK0));
+                        }
+                        f16x2 const p01 = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(p[0], p[1]));
+                        f16x2 const p23 = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(p[2], p[3]));
+                        preg[w * 4 + 0] = p01[0];
+                        preg[w * 4 + 1] = p01[1];
+                        preg[w * 4 + 2] = p23[0];
+                        preg[w * 4 + 3] = p23[1];
+                    }
+                    // V^T operand: lane r of a group addresses LDS row (4 keys per read: r/4) at
+                    // halfword 16dt + 4(r%4); the transpose read hands lane i the 4 keys of head
+                    // dim 16dt + i.  Slots 0..3 = keys 16(2hb)+4g.., slots 4..7 = keys 16(2hb+1)+4g..
+                    int const vrow = kb * 64 + hb * 32 + 4 * g + (lq >> 2);
+                    uint8_t const* vbase = sV + vrow * kRow + 8 * (lq & 1);
+#pragma unroll
+                    for (int dt = 0; dt < 4; ++dt)
+                    {
+                        // rows vrow and vrow + 16 share row & 7, hence the swizzled chunk
+                        int const sc = swz<2>(vrow, 2 * dt + ((lq >> 1) & 1)) * 16;
+                        i16x4 const v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vbase + sc));
+                        i16x4 const v1
+                            = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vbase + 16 * kRow + sc));
+                        typedef short i16x8 __attribute__((ext_vector_type(8)));
+                        i16x8 const both = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            __builtin_bit_cast(f16x8, both), preg, oacc[dt], 0, 0, 0);
+                    }
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, preg, sacc, 0, 0, 0);
+                }
             }
-            int const d0 = dt * 16 + g * 4;
-            int64_t const off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + d0) * 2;
-            *reinterpret_cast<u32x2*>(dst + off) = __builtin_bit_cast(u32x2, y);
+        }
+
+        if (qValid)
+        {
+            float const rinv = sacc[0] > 0.f ? 1.f / sacc[0] : 0.f;
+            uint8_t* dst = static_cast<uint8_t*>(a.out);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+            {
+                f16x4 y;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    y[j] = (f16) (oacc[dt][j] * rinv);
+                }
+                int const d0 = dt * 16 + g * 4;
+                int64_t const off
+                    = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + d0) * 2;
+                *reinterpret_cast<u32x2*>(dst + off) = __builtin_bit_cast(u32x2, y);
+            }
         }
     }
 }
@@ -723,7 +843,7 @@ int launch_fmha(K kernel, char const* name, hipStream_t stream, FmhaArgs const& 
             done.push_back(key);
         }
     }
-    unsigned const blocks = (unsigned) args.B * args.N * args.qTiles;
+    unsigned const blocks = (unsigned) args.B * args.N * args.qSplit;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWaveSize), ldsBytes, stream, args);
     return check_launch(name);
 }
@@ -853,7 +973,28 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
     a.B = p->b;
     a.N = p->h;
     a.S = p->s;
-    a.qTiles = ceil_div(p->s, (dataType == 2 ? kWavesI8 : kWavesF16) * kQPerWave);
+    {
+        // Workgroups per (sequence, head): one, unless the launch would leave compute units idle
+        // (fewer than ~4 workgroups per CU) and the rows are long enough to share.
+        int const waves = dataType == 2 ? kWavesI8 : kWavesF16;
+        int const maxSplit = std::max(1, ceil_div(ceil_div(p->s, kQPerWave), waves));
+        int64_t const heads = (int64_t) p->b * p->h;
+        int split = 1;
+        while (split < maxSplit && heads * split < 1024)
+        {
+            split *= 2;
+        }
+        a.qSplit = std::min(split, maxSplit);
+        // tuning override: TRTAMD_FMHA_QSPLIT=<n> forces the number of workgroups per head
+        static int const forced = [] {
+            char const* e = getenv("TRTAMD_FMHA_QSPLIT");
+            return e ? atoi(e) : 0;
+        }();
+        if (forced > 0)
+        {
+            a.qSplit = std::min(forced, maxSplit);
+        }
+    }
     a.dbgAcc1 = dbgAcc1;
     a.dbgP8 = dbgP8;
     if (interleaved)

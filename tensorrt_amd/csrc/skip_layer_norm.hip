@@ -378,12 +378,6 @@ __global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const to
     constexpr bool RESIDENT = NI <= 8;
     __shared__ float sGamma[LD];
     __shared__ float sBeta[LD];
-    for (int i = threadIdx.x; i < LD; i += kBlock)
-    {
-        sGamma[i] = (float) gamma[i] * qScale;
-        sBeta[i] = (float) beta[i] * qScale;
-    }
-    __syncthreads();
 
     int const lane = threadIdx.x & (kWaveSize - 1);
     int const sub = lane >> 4;
@@ -439,6 +433,13 @@ __global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const to
             }
         }
     }
+    // gamma/beta are staged after the tensor loads were issued, so their latency overlaps
+    for (int i = threadIdx.x; i < LD; i += kBlock)
+    {
+        sGamma[i] = (float) gamma[i] * qScale;
+        sBeta[i] = (float) beta[i] * qScale;
+    }
+    __syncthreads();
     // the 8 lanes of a token differ in bit 0 (half) and bits 4,5 (sub)
 #pragma unroll
     for (int m : {1, 16, 32})
