@@ -9,9 +9,14 @@
  * Each function cites the reference source it follows (paths relative to the reference root).
  *
  * What a CPU restatement cannot restate, and therefore leaves PARITY UNPINNED at bit level:
- *   - the summation order of cub::BlockReduce (CCCL v3.4.0-rc0, fetched at configure time by
- *     cmake/modules/FetchCCCL.cmake:22, absent from the checkout).  Per-thread partial sums are
- *     formed exactly as the kernels form them; the partials are then added in thread order.
+ *   - cub::BlockReduce lives in CCCL (v3.4.0-rc0, fetched at configure time by
+ *     cmake/modules/FetchCCCL.cmake:22, absent from the checkout).  Its published default algorithm
+ *     (BLOCK_REDUCE_WARP_REDUCTIONS) is restated in block_reduce_pair below: a shuffle-down tree
+ *     inside every 32-lane warp, then lane 0 adds the warp aggregates in warp order.  Per-thread
+ *     partial sums are formed exactly as the kernels form them.  Whether the installed CCCL build
+ *     specialises differently for a given type is not checkable here, so binary16 LayerNorm
+ *     statistics stay unpinned at bit level (they are pinned to float64 within binary16 accuracy).
+ *     The binary32 softmax sums are added in index order (differences of a few ulp).
  *   - the inside of the fused-attention cubins (SASS only).  Rounding is fixed here as
  *     round-to-nearest-even with saturation to [-128,127], softmax in binary32.
  *   - cuBLAS binary16 GEMM accumulation order/width in the unfused path
@@ -206,6 +211,48 @@ static inline float t_rsqrt(int is_half, float a)
 }
 
 /*
+ * cub::BlockReduce<T, TPB>::Reduce with the default BLOCK_REDUCE_WARP_REDUCTIONS algorithm, for a
+ * pair of values reduced together (kvp<T> / half2 with a component-wise sum), TPB a multiple of 32:
+ *   inside each warp, for offset = 1, 2, 4, 8, 16: lane l adds the value lane l+offset held before
+ *   the step (when l+offset < 32); lane 0 ends with the warp aggregate;
+ *   thread 0 then adds the aggregates of warps 1, 2, ... to its own, in that order.
+ */
+static void block_reduce_pair(int is_half, int nthreads, float const* p1, float const* p2, float* o1, float* o2)
+{
+    float tot1 = 0.f, tot2 = 0.f;
+    for (int w0 = 0; w0 < nthreads; w0 += 32)
+    {
+        float a[32], b[32];
+        int nl = nthreads - w0 < 32 ? nthreads - w0 : 32;
+        for (int l = 0; l < 32; ++l)
+        {
+            a[l] = l < nl ? p1[w0 + l] : 0.f;
+            b[l] = l < nl ? p2[w0 + l] : 0.f;
+        }
+        for (int off = 1; off < 32; off <<= 1)
+        {
+            for (int l = 0; l + off < nl; ++l) /* ascending l reads lanes not yet updated in this step */
+            {
+                a[l] = t_add(is_half, a[l], a[l + off]);
+                b[l] = t_add(is_half, b[l], b[l + off]);
+            }
+        }
+        if (w0 == 0)
+        {
+            tot1 = a[0];
+            tot2 = b[0];
+        }
+        else
+        {
+            tot1 = t_add(is_half, tot1, a[0]);
+            tot2 = t_add(is_half, tot2, b[0]);
+        }
+    }
+    *o1 = tot1;
+    *o2 = tot2;
+}
+
+/*
  * One row of computeSkipLayerNorm<T,hasBias>.
  * Dispatch (skipLayerNormKernel.cu:261-282): ld<=32 -> skipLayerNormKernelSmall (one element per
  * thread, no epsilon); ld in {768,1024} -> skipln_vec (VPT = 16/sizeof(T) consecutive elements
@@ -260,12 +307,8 @@ static void skipln_row(int is_half, int ld, float const* in, float const* skip, 
             part2[t] = t_add(is_half, part2[t], t_mul(is_half, tmp, v));
         }
     }
-    float mu = 0.f, m2 = 0.f;
-    for (int t = 0; t < nthreads; ++t)
-    {
-        mu = t_add(is_half, mu, part1[t]);
-        m2 = t_add(is_half, m2, part2[t]);
-    }
+    float mu, m2;
+    block_reduce_pair(is_half, nthreads, part1, part2, &mu, &m2);
     float var = t_sub(is_half, m2, t_mul(is_half, mu, mu));
     if (vec)
     {
@@ -335,7 +378,7 @@ static void dqq_half_core(int ld, float const* v /* binary16 values */, float co
 {
     float const rld = hr(1.0 / (double) hr((double) ld));
     int nthreads = ld / 8;
-    float mu = 0.f, m2 = 0.f;
+    float part1[512], part2[512];
     for (int t = 0; t < nthreads; ++t)
     {
         float p1 = 0.f, p2 = 0.f;
@@ -346,9 +389,11 @@ static void dqq_half_core(int ld, float const* v /* binary16 values */, float co
             p1 = hr((double) p1 + tmp);
             p2 = hr((double) p2 + hr((double) tmp * x));
         }
-        mu = hr((double) mu + p1);
-        m2 = hr((double) m2 + p2);
+        part1[t] = p1;
+        part2[t] = p2;
     }
+    float mu, m2;
+    block_reduce_pair(1, nthreads, part1, part2, &mu, &m2);
     float var = hr((double) hr((double) m2 - hr((double) mu * mu)) + 0.0009765625);
     float rsigma;
     if (rsqrt_in_float)
@@ -599,12 +644,8 @@ static int embln_token(int is_half, int ld, int32_t wordId, int32_t tokenId, int
         part1[t] = t_add(is_half, part1[t], rv);
         part2[t] = t_add(is_half, part2[t], t_mul(is_half, rv, v));
     }
-    float mu = 0.f, m2 = 0.f;
-    for (int t = 0; t < 256; ++t)
-    {
-        mu = t_add(is_half, mu, part1[t]);
-        m2 = t_add(is_half, m2, part2[t]);
-    }
+    float mu, m2;
+    block_reduce_pair(is_half, 256, part1, part2, &mu, &m2);
     float rsigma = t_rsqrt(is_half, t_sub(is_half, m2, t_mul(is_half, mu, mu)));
     for (int i = 0; i < ld; ++i)
     {

@@ -3,7 +3,7 @@
 The product is ``lib/libtrtamd_bert_plugins.so``: hand-written gfx950 kernels behind a C ABI
 (``include/trtamd_bert_kernels.h``) and the IPluginV3 host classes registered under the reference's
 plugin names.  This package is the thin Python side: it locates and loads that library and exposes
-ctypes bindings (``tensorrt_amd.capi``) plus a plugin-level driver (``tensorrt_amd.plugin_api``).
+ctypes bindings (``tensorrt_amd.capi``) plus a plugin-level driver (``tensorrt_amd.plugin``).
 There is no CPU fallback: if the library is missing, loading raises.
 """
 from __future__ import annotations

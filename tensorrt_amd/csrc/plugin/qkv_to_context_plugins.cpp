@@ -355,7 +355,12 @@ protected:
             p.d = mHeadSize;
             p.qkv_stride_in_bytes = int64_t(3) * mB * mNumHeads * mHeadSize * esize; // mLdQKV
             p.o_stride_in_bytes = int64_t(mB) * mNumHeads * mHeadSize * esize;       // mLdOut
-            p.packed_mask_stride_in_bytes = int64_t(getMHAMaskPackedSize(mSM, mType, mS)) * 4;
+            // The embedding plugin sizes the mask tensor for S = 128 but packs S = 64 and 96 densely:
+            // the per-sequence stride is xmmas_m * threads words (mhaRunner.cu:676-697, 818-831)
+            int32_t const warpsM = mS == 384 ? 1 : 2;
+            int32_t const threads = mS == 384 ? 256 : 128;
+            int32_t const xmmasM = (mS + 16 * warpsM - 1) / (16 * warpsM);
+            p.packed_mask_stride_in_bytes = int64_t(xmmasM) * threads * 4;
             float const rsqrtHead = 1.F / std::sqrt(static_cast<float>(mHeadSize));
             if (mType == DataType::kINT8)
             {

@@ -1,0 +1,92 @@
+"""GPU parity of the unfused attention path (scaled/masked softmax, strided batched GEMMs) and of
+zeroPadding2d, through the C ABI."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_fp_close, attention_f64, dev, dev_empty, host, ptr, rng, stream, sync
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def api():
+    from tensorrt_amd import capi
+    return capi.api()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("S,masked", [(16, True), (128, True), (384, False), (100, True), (1000, True), (33, False)])
+def test_scaled_softmax(api, dt, S, masked):
+    r = rng(200 + S)
+    B, N = 3, 2
+    x = (3 * r.standard_normal((B, N, S, S))).astype(dt)
+    lens = np.array([S, 1, max(1, S // 3)], np.int32) if masked else None
+    out = dev_empty((B, N, S, S), dt, fill=1)
+    fn = api.scaled_softmax_fp32 if dt == np.float32 else api.scaled_softmax_fp16
+    d_len = dev(lens) if masked else None
+    api.check(fn(stream(), S, B, N, 0.125, ptr(d_len), ptr(dev(x)), ptr(out)))
+    sync()
+    got = host(out)
+    ref = oracle.scaled_softmax(x, 0.125, lens)
+    assert_fp_close(got, ref, atol=1e-5 if dt == np.float32 else 1e-3, rtol=1e-4 if dt == np.float32 else 2e-3,
+                    what="softmax")
+    if masked:
+        for b in range(B):
+            assert not got[b][..., lens[b]:].any()      # masked positions are exactly zero
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("S,B,N,d,masked", [(128, 2, 12, 64, True), (20, 3, 2, 32, True), (77, 1, 3, 48, False),
+                                            (384, 1, 2, 64, True), (5, 2, 1, 8, False), (130, 2, 2, 128, True)])
+def test_unfused_mha(api, dt, S, B, N, d, masked):
+    r = rng(210 + S + d)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
+    lens = r.integers(1, S + 1, B).astype(np.int32) if masked else None
+    type_id = 0 if dt == np.float32 else 1
+    ws_bytes = api.unfused_mha_workspace_size(type_id, S, B, N)
+    ws = dev_empty((ws_bytes,), np.uint8)
+    out = dev_empty((S, B, N * d), dt, fill=0)
+    d_len = dev(lens) if masked else None
+    api.check(api.unfused_mha(stream(), type_id, S, B, N, d, ptr(dev(qkv)), ptr(d_len), ptr(out), ptr(ws)))
+    sync()
+    got = host(out)
+    ref = oracle.mha_unfused_fixed(qkv, S, B, N, d, lens)
+    tol = dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}
+    assert_fp_close(got, ref, what="vs oracle", **tol)
+    # and against float64 attention for one (sequence, head)
+    t = qkv.reshape(S, B, N, 3, d)
+    L = int(lens[0]) if masked else S
+    closed = attention_f64(t[:, 0, 0, 0], t[:L, 0, 0, 1], t[:L, 0, 0, 2], 1 / np.sqrt(d))
+    assert_fp_close(got.reshape(S, B, N, d)[:, 0, 0], closed, what="vs float64",
+                    **(dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else dict(atol=4e-3, rtol=1e-2)))
+
+
+def test_unfused_mha_rejects_int8(api):
+    assert api.unfused_mha(None, 2, 16, 1, 1, 64, 0, 0, 0, 0) != 0
+    assert "data type" in api.last_error_str()
+
+
+@pytest.mark.parametrize("spitch,dpitch,height", [(64, 128, 1000), (80, 128, 7), (32, 64, 333), (128, 64, 50),
+                                                  (64, 64, 9), (2, 64, 5)])
+def test_zero_padding_2d(api, spitch, dpitch, height):
+    r = rng(220 + spitch)
+    src = r.integers(0, 256, height * spitch).astype(np.uint8)
+    dst = dev_empty((height * dpitch,), np.uint8, fill=0xAB)
+    api.check(api.zero_padding_2d(ptr(dev(src)), spitch, ptr(dst), dpitch, height, stream()))
+    sync()
+    assert np.array_equal(host(dst), oracle.zero_padding_2d(src, spitch, dpitch, height))
+
+
+def test_zero_padding_round_trip_at_attention_size(api):
+    """Pad [T,N,3,32] to head size 64 and strip it again: identity."""
+    T, N = 2048, 16
+    src = rng(221).integers(0, 256, T * N * 3 * 32 * 2).astype(np.uint8)   # binary16 elements
+    rows = T * N * 3
+    mid = dev_empty((rows * 128,), np.uint8)
+    back = dev_empty((rows * 64,), np.uint8)
+    api.check(api.zero_padding_2d(ptr(dev(src)), 64, ptr(mid), 128, rows, stream()))
+    api.check(api.zero_padding_2d(ptr(mid), 128, ptr(back), 64, rows, stream()))
+    sync()
+    assert np.array_equal(host(back), src)
+    assert not host(mid).reshape(rows, 128)[:, 64:].any()

@@ -1,0 +1,84 @@
+"""The shared library loads without a GPU and exports every symbol the headers declare.
+No compute entry point is called here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import tensorrt_amd
+from tensorrt_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INCLUDE = os.path.join(ROOT, "include")
+
+
+def _declared(header, macro):
+    text = open(os.path.join(INCLUDE, header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    text = re.sub(r"^\s*#[^\n]*", "", text, flags=re.M)
+    names = re.findall(macro + r"\s+[^;{(]*?\b(\w+)\s*\(", text)
+    return sorted(set(names))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return tensorrt_amd.load_library()
+
+
+def test_kernel_header_symbols_exported(lib):
+    names = _declared("trtamd_bert_kernels.h", "TRTAMD_API")
+    assert len(names) >= 24
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in trtamd_bert_kernels.h but not exported"
+    # the ctypes table covers the same set
+    assert sorted(capi.HEADER_SYMBOLS) == names
+
+
+def test_plugin_c_header_symbols_exported(lib):
+    from tensorrt_amd import plugin
+    names = _declared("trtamd_plugin_c.h", "TRTAMD_PLUGIN_API")
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in trtamd_plugin_c.h but not exported"
+    assert sorted(plugin.plugin_c_symbols()) == names
+
+
+def test_nvinfer_entry_points_exported(lib):
+    names = _declared("trtamd_nvinfer_api.h", r'extern\s+"C"\s+TENSORRTAPI')
+    assert set(names) == {"getPluginRegistry", "getLogger", "initLibNvInferPlugins", "setLoggerFinder", "getCreators"}
+    for n in names:
+        assert hasattr(lib, n)
+
+
+def test_version_and_error_string(lib):
+    a = capi.api()
+    assert a.version() >= 1
+    assert isinstance(a.last_error_str(), str)
+
+
+def test_fused_kernel_validity_table():
+    a = capi.api()
+    for dtype in (1, 2):
+        for s in (1, 64, 96, 128, 192, 256, 384, 512):
+            assert a.fused_mha_is_valid(dtype, 64, s) == 1
+        assert a.fused_mha_is_valid(dtype, 64, 513) == 0
+        assert a.fused_mha_is_valid(dtype, 32, 128) == 0
+        assert a.fused_mha_is_valid(dtype, 128, 128) == 0
+    assert a.fused_mha_is_valid(0, 64, 128) == 0  # no fused kernel in binary32
+
+
+def test_unfused_workspace_formula():
+    a = capi.api()
+    # two S x S score matrices per (batch, head) in the compute type (mhaRunner.cu:522-525)
+    assert a.unfused_mha_workspace_size(0, 128, 2, 12) == 2 * 4 * 128 * 128 * 2 * 12
+    assert a.unfused_mha_workspace_size(1, 384, 1, 16) == 2 * 2 * 384 * 384 * 16
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    """No fallback: without the built library the package raises."""
+    monkeypatch.setattr(tensorrt_amd, "_handle", None)
+    monkeypatch.setattr(tensorrt_amd, "_LIB", str(tmp_path / "nope.so"))
+    with pytest.raises(tensorrt_amd.LibraryNotBuilt):
+        tensorrt_amd.load_library()
