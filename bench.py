@@ -83,7 +83,7 @@ def cpu_baseline(wl, s_ctx, s_out, budget_s=20.0):
         assert st == 0
         reps += 1
         el = time.perf_counter() - t0
-        if el > budget_s / 2 or reps >= 3:
+        if el > budget_s:
             break
     return {"value": round(nseq * reps / el, 3), "unit": "sequences/s", "cores": threads, "kind": "port",
             "sample": f"{reps} pass(es) over the first {nseq} of {wl.B} sequences ({T} tokens): C oracle "
@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--seqlen", type=int, default=384)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain elementwise copy of known size (256 MiB read + 256 MiB written), the "
+                         "yardstick FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every sequence, head and LayerNorm row "
@@ -133,23 +136,43 @@ def main():
                                                       d["beta"].data_ptr(), d["gamma"].data_ptr(), d["out"].data_ptr(),
                                                       s_ctx, wl.s_skip, q_out))
 
-    for _ in range(args.warmup):
+    def step():
         mha()
         skipln()
+
+    for _ in range(max(args.warmup, 1)):
+        step()
     torch.cuda.synchronize()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        ev[i][0].record()
-        mha()
-        ev[i][1].record()
-        skipln()
-        ev[i][2].record()
+    for _ in range(args.steps):
+        step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_step = wall * 1e3 / args.steps
-    t_mha = float(np.mean([e[0].elapsed_time(e[1]) for e in ev])) * 1e-3
-    t_ln = float(np.mean([e[1].elapsed_time(e[2]) for e in ev])) * 1e-3
+
+    # Per-kernel durations for the roofline records, outside the timed region: each kernel launched
+    # back to back `steps` times between two events on the stream it runs on (an event pair around a
+    # single 20-60 us launch would add its own few microseconds to every sample).
+    def kernel_time(fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / args.steps
+
+    t_mha = kernel_time(mha)
+    t_ln = kernel_time(skipln)
+
+    if args.pmc_calibration:
+        src = torch.zeros(256 << 20, dtype=torch.int8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
 
     mha_ops = wl.mha_ops()
     ln_bytes = wl.skipln_bytes(1)
