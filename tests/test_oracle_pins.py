@@ -402,3 +402,79 @@ def test_fused_int8_fixed_and_packed_agree():
         ln = int(lens[b])
         packed = oracle.mha_fused_i8_packed(qkv[:ln, b], np.array([0, ln], np.int32), N, d, *sc)
         assert np.array_equal(fixed[:ln, b], packed)
+
+
+def test_packed_mask_all_contiguous_lengths():
+    """Every prefix length 0..S for the four sequence lengths that have a packed mask: decoding
+    (by the fragment layout above, vectorised) gives back `col < len` everywhere."""
+    for S, wm, wn in ((64, 2, 2), (96, 2, 2), (128, 2, 2), (384, 1, 8)):
+        lens = np.arange(S + 1)
+        mask = (np.arange(S)[:, None] < lens[None, :]).astype(np.int32)
+        packed, over = oracle.convert_mask(mask, wm, wn)
+        assert over == 0
+        xm, xn, threads = oracle.packed_mask_geometry(S, wm, wn)
+        t = np.arange(threads)
+        warp_n, lane = (t // 32) // wm, t % 32
+        col_off = np.array([0, 1, 0, 1, 8, 9, 8, 9])
+        # column of bit (ni, k) of thread t
+        col = ((np.arange(xn)[None, :, None] * wn + warp_n[:, None, None]) * 16 + 2 * (lane % 4)[:, None, None]
+               + col_off[None, None, :])                                        # [threads, xn, 8]
+        shift = (8 * np.arange(xn)[:, None] + np.arange(8)[None, :])[None]       # [1, xn, 8]
+        words = packed.reshape(S + 1, xm, threads)
+        bits = (words[..., None, None] >> shift[None]) & 1                       # [S+1, xm, threads, xn, 8]
+        want = col[None, None] < lens[:, None, None, None, None]
+        assert np.array_equal(bits.astype(bool), np.broadcast_to(want, bits.shape))
+
+
+def test_attention_special_cases():
+    r = rng(90)
+    N, d = 2, 64
+    # a sequence of one token attends only itself: the context is V
+    qkv = r.standard_normal((1, 3 * N * d)).astype(np.float16)
+    out = oracle.mha_fused_f16_packed(qkv, np.array([0, 1], np.int32), N, d)
+    assert np.array_equal(out, qkv.reshape(1, N, 3, d)[:, :, 2].reshape(1, N * d))
+    # identical keys give uniform probabilities: the context is the mean of V, for every query
+    L = 16
+    qkv = r.standard_normal((L, N, 3, d)).astype(np.float32)
+    qkv[:, :, 1] = qkv[0, :, 1]
+    got = oracle.mha_unfused_fixed(qkv.reshape(L, 1, 3 * N * d), L, 1, N, d).reshape(L, N, d)
+    close(got, np.broadcast_to(qkv[:, :, 2].mean(0), (L, N, d)), atol=1e-5, rtol=1e-5)
+    # INT8, one token: p8 = 127 exactly, context = sat(rne(127 * v * scale_bmm2))
+    q8 = r.integers(-127, 128, (1, 3 * N * d)).astype(np.int8)
+    s2 = np.float32(0.006)
+    o8, a1, p8, a2 = oracle.mha_fused_i8_packed(q8, np.array([0, 1], np.int32), N, d, np.float32(1e-4),
+                                                np.float32(127.0), s2, want_ints=True)
+    v = q8.reshape(1, N, 3, d)[:, :, 2].astype(np.int64)
+    assert (p8[:, :, 0, 0] == 127).all()
+    assert np.array_equal(a2.reshape(1, N, d), 127 * v)
+    assert np.array_equal(o8.reshape(1, N, d), np.clip(np.rint((127 * v).astype(np.float32) * s2), -128, 127))
+    # packing invariance: a sequence computes the same alone or inside a batch
+    lens = np.array([5, 12, 7])
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    x = r.integers(-127, 128, (int(cu[-1]), 3 * N * d)).astype(np.int8)
+    sc = (np.float32(2e-4), np.float32(127.0), np.float32(0.01))
+    whole = oracle.mha_fused_i8_packed(x, cu, N, d, *sc)
+    for b in range(3):
+        alone = oracle.mha_fused_i8_packed(x[cu[b]:cu[b + 1]], np.array([0, lens[b]], np.int32), N, d, *sc)
+        assert np.array_equal(whole[cu[b]:cu[b + 1]], alone)
+
+
+def test_int8_layernorm_all_byte_pairs():
+    """Every (input, skip) byte pair appears in one hidden vector: the dequantised sum the oracle
+    normalises is exactly dqIn*a + dqSkip*b for all 65536 pairs (checked through the Megatron
+    variant's pre-LayerNorm output, quantised with scale 1)."""
+    a = np.arange(-128, 128, dtype=np.int16)
+    pairs = np.stack(np.meshgrid(a, a, indexing="ij"), -1).reshape(-1, 2).astype(np.int8)   # 65536 pairs
+    ld = 1024
+    total = pairs.shape[0] // ld                                                           # 64 tokens
+    x = pairs[:, 0].reshape(total, ld)
+    s = pairs[:, 1].reshape(total, ld)
+    gamma = np.ones(ld, np.float16)
+    beta = np.zeros(ld, np.float16)
+    for force, lo in ((0, -127), (1, -128)):
+        st, _, pre = oracle.skipln_interleaved(1, oracle.interleave(x), oracle.interleave(s), beta, gamma, ld, total,
+                                               0.5, 0.25, 1.0, 1.0, force=force)
+        assert st == 0
+        want = np.clip(np.rint(0.5 * x.astype(np.float64) + 0.25 * s.astype(np.float64)), lo, 127)
+        # .5 ties: 0.5*a + 0.25*b is exact in binary16/32, so round-half-even decides identically
+        assert np.array_equal(oracle.deinterleave(pre, total, ld), want.astype(np.int8))
