@@ -12,6 +12,8 @@
 #include "device_utils.hpp"
 #include "host_utils.hpp"
 
+#include <cstdlib>
+
 namespace trtamd
 {
 namespace
@@ -367,88 +369,100 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
 // in*skip, sum skip^2) combined in binary64, so mean and variance carry no accumulation error.
 // gamma*qScale and beta*qScale are staged once per workgroup in LDS as binary32.
 // ------------------------------------------------------------------------------------------
-template <int G, bool PRELN>
-__global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const total, int8_t const* __restrict__ in,
-    int8_t const* __restrict__ skip, f16 const* __restrict__ beta, f16 const* __restrict__ gamma,
-    int8_t* __restrict__ out, int8_t* __restrict__ preln, float const dqIn, float const dqSkip, float const qScale,
-    float const qSkipScale, float const eps, float const prelnMin)
+template <int G, int W, int TOK, bool PRELN>
+__global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int const total,
+    int8_t const* __restrict__ in, int8_t const* __restrict__ skip, f16 const* __restrict__ beta,
+    f16 const* __restrict__ gamma, int8_t* __restrict__ out, int8_t* __restrict__ preln, float const dqIn,
+    float const dqSkip, float const qScale, float const qSkipScale, float const eps, float const prelnMin)
 {
+    // A workgroup of W wavefronts owns TOK consecutive tokens.  Lane = (sub, token, half): one load
+    // instruction of a wavefront reads SUBS channel groups x TOK tokens x 32 bytes, TOK*32 contiguous
+    // bytes per group; the W wavefronts take interleaved sets of SUBS groups, NI sets each.
     constexpr int LD = G * 32;
-    constexpr int NI = G / 4;
-    constexpr bool RESIDENT = NI <= 8;
+    constexpr int THREADS = W * kWaveSize;
+    constexpr int LPG = TOK * 2;               // lanes per channel group
+    constexpr int SUBS = kWaveSize / LPG;      // channel groups per load instruction
+    constexpr int NI = G / (SUBS * W);
+    static_assert(G % (SUBS * W) == 0 && NI <= 8, "every lane keeps its part of the row in registers");
     __shared__ float sGamma[LD];
     __shared__ float sBeta[LD];
+    __shared__ int sStat[W][TOK][5];
 
     int const lane = threadIdx.x & (kWaveSize - 1);
-    int const sub = lane >> 4;
-    int const tok = (lane & 15) >> 1;
+    int const wave = threadIdx.x >> 6;
+    int const sub = lane / LPG;
+    int const tok = (lane % LPG) >> 1;
     int const hf = lane & 1;
-    int64_t const t = ((int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * 8 + tok;
-    bool const valid = t < total;
+    int64_t const tRaw = (int64_t) blockIdx.x * TOK + tok;
+    bool const valid = tRaw < total;
+    // lanes past the last token re-read the last token (and store nothing): no divergent loads
+    int64_t const t = valid ? tRaw : (int64_t) total - 1;
     int64_t const groupStride = (int64_t) total * 32;
-    int64_t const base = (int64_t) sub * groupStride + t * 32 + hf * 16;
+    int const g0 = wave * SUBS + sub;               // first channel group of this lane; then += SUBS*W
+    int64_t const base = (int64_t) g0 * groupStride + t * 32 + hf * 16;
+    constexpr int64_t kStep = SUBS * W;
 
-    u32x4 xi[RESIDENT ? NI : 1], xs[RESIDENT ? NI : 1];
-    int sIn = 0, sSk = 0, sII = 0, sIS = 0, sSS = 0;
+    u32x4 xi[NI], xs[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i)
     {
-        u32x4 a = {0, 0, 0, 0}, s = {0, 0, 0, 0};
-        if (valid)
-        {
-            a = *reinterpret_cast<u32x4 const*>(in + base + (int64_t) i * 4 * groupStride);
-            s = *reinterpret_cast<u32x4 const*>(skip + base + (int64_t) i * 4 * groupStride);
-        }
-        if (RESIDENT)
-        {
-            xi[i] = a;
-            xs[i] = s;
-        }
-        else
-        {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                sIn = __builtin_amdgcn_sdot4((int) a[q], 0x01010101, sIn, false);
-                sSk = __builtin_amdgcn_sdot4((int) s[q], 0x01010101, sSk, false);
-                sII = __builtin_amdgcn_sdot4((int) a[q], (int) a[q], sII, false);
-                sIS = __builtin_amdgcn_sdot4((int) a[q], (int) s[q], sIS, false);
-                sSS = __builtin_amdgcn_sdot4((int) s[q], (int) s[q], sSS, false);
-            }
-        }
-    }
-    if (RESIDENT)
-    {
-#pragma unroll
-        for (int i = 0; i < NI; ++i)
-        {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                sIn = __builtin_amdgcn_sdot4((int) xi[i][q], 0x01010101, sIn, false);
-                sSk = __builtin_amdgcn_sdot4((int) xs[i][q], 0x01010101, sSk, false);
-                sII = __builtin_amdgcn_sdot4((int) xi[i][q], (int) xi[i][q], sII, false);
-                sIS = __builtin_amdgcn_sdot4((int) xi[i][q], (int) xs[i][q], sIS, false);
-                sSS = __builtin_amdgcn_sdot4((int) xs[i][q], (int) xs[i][q], sSS, false);
-            }
-        }
+        xi[i] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(in + base + i * kStep * groupStride));
+        xs[i] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(skip + base + i * kStep * groupStride));
     }
     // gamma/beta are staged after the tensor loads were issued, so their latency overlaps
-    for (int i = threadIdx.x; i < LD; i += kBlock)
+    for (int i = threadIdx.x; i < LD; i += THREADS)
     {
         sGamma[i] = (float) gamma[i] * qScale;
         sBeta[i] = (float) beta[i] * qScale;
     }
-    __syncthreads();
-    // the 8 lanes of a token differ in bit 0 (half) and bits 4,5 (sub)
+    int sIn = 0, sSk = 0, sII = 0, sIS = 0, sSS = 0;
 #pragma unroll
-    for (int m : {1, 16, 32})
+    for (int i = 0; i < NI; ++i)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            sIn = __builtin_amdgcn_sdot4((int) xi[i][q], 0x01010101, sIn, false);
+            sSk = __builtin_amdgcn_sdot4((int) xs[i][q], 0x01010101, sSk, false);
+            sII = __builtin_amdgcn_sdot4((int) xi[i][q], (int) xi[i][q], sII, false);
+            sIS = __builtin_amdgcn_sdot4((int) xi[i][q], (int) xs[i][q], sIS, false);
+            sSS = __builtin_amdgcn_sdot4((int) xs[i][q], (int) xs[i][q], sSS, false);
+        }
+    }
+    // the lanes of a token differ in bit 0 (half) and in the sub bits above the token bits
+#pragma unroll
+    for (int m = 1; m < kWaveSize; m = (m == 1 ? LPG : m * 2))
     {
         sIn += __shfl_xor(sIn, m, kWaveSize);
         sSk += __shfl_xor(sSk, m, kWaveSize);
         sII += __shfl_xor(sII, m, kWaveSize);
         sIS += __shfl_xor(sIS, m, kWaveSize);
         sSS += __shfl_xor(sSS, m, kWaveSize);
+    }
+    if (W > 1)
+    {
+        if (sub == 0 && hf == 0)
+        {
+            sStat[wave][tok][0] = sIn;
+            sStat[wave][tok][1] = sSk;
+            sStat[wave][tok][2] = sII;
+            sStat[wave][tok][3] = sIS;
+            sStat[wave][tok][4] = sSS;
+        }
+    }
+    __syncthreads();
+    if (W > 1)
+    {
+        sIn = sSk = sII = sIS = sSS = 0;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+        {
+            sIn += sStat[w][tok][0];
+            sSk += sStat[w][tok][1];
+            sII += sStat[w][tok][2];
+            sIS += sStat[w][tok][3];
+            sSS += sStat[w][tok][4];
+        }
     }
     double const dIn = (double) dqIn, dSk = (double) dqSkip;
     double const mean = (dIn * sIn + dSk * sSk) * (1.0 / LD);
@@ -467,23 +481,8 @@ __global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const to
 #pragma unroll
     for (int i = 0; i < NI; ++i)
     {
-        u32x4 a, s;
-        if (RESIDENT)
-        {
-            a = xi[i];
-            s = xs[i];
-        }
-        else
-        {
-            a = u32x4{0, 0, 0, 0};
-            s = u32x4{0, 0, 0, 0};
-            if (valid)
-            {
-                a = *reinterpret_cast<u32x4 const*>(in + base + (int64_t) i * 4 * groupStride);
-                s = *reinterpret_cast<u32x4 const*>(skip + base + (int64_t) i * 4 * groupStride);
-            }
-        }
-        int const ch = (i * 4 + sub) * 32 + hf * 16;
+        u32x4 const a = xi[i], s = xs[i];
+        int const ch = (g0 + i * (int) kStep) * 32 + hf * 16;
         u32x4 o, po;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
@@ -504,9 +503,9 @@ __global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const to
                 yb[k] = __float_as_uint(y + kMagic);
                 if (PRELN)
                 {
-                    float p = fmaf(fa, p1, fmaf(fs, p2, pc));
-                    p = __builtin_amdgcn_fmed3f(p, prelnMin, 127.f);
-                    pb[k] = __float_as_uint(p + kMagic);
+                    float pv = fmaf(fa, p1, fmaf(fs, p2, pc));
+                    pv = __builtin_amdgcn_fmed3f(pv, prelnMin, 127.f);
+                    pb[k] = __float_as_uint(pv + kMagic);
                 }
             }
             uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
@@ -521,29 +520,34 @@ __global__ __launch_bounds__(kBlock) void skipln_interleaved_kernel(int const to
         }
         if (valid)
         {
-            *reinterpret_cast<u32x4*>(out + base + (int64_t) i * 4 * groupStride) = o;
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + base + i * kStep * groupStride));
             if (PRELN)
             {
-                *reinterpret_cast<u32x4*>(preln + base + (int64_t) i * 4 * groupStride) = po;
+                __builtin_nontemporal_store(po, reinterpret_cast<u32x4*>(preln + base + i * kStep * groupStride));
             }
         }
     }
 }
 
-template <int G>
+template <int G, int W, int TOK>
 int launch_interleaved(hipStream_t stream, int32_t total, int8_t const* in, int8_t const* skip, f16 const* beta,
     f16 const* gamma, int8_t* out, int8_t* preln, float dqIn, float dqSkip, float qScale, float qSkipScale, float eps,
     float prelnMin)
 {
-    dim3 const grid((unsigned) ceil_div(total, 8 * kWavesPerBlock));
+    dim3 const grid((unsigned) ceil_div(total, TOK));
+    dim3 const block(W * kWaveSize);
+    static int const dynLds = [] {
+        char const* e = getenv("TRTAMD_SKIPLN_LDS");
+        return e ? atoi(e) : 0;
+    }();
     if (preln)
     {
-        hipLaunchKernelGGL((skipln_interleaved_kernel<G, true>), grid, dim3(kBlock), 0, stream, total, in, skip, beta,
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, true>), grid, block, 0, stream, total, in, skip, beta,
             gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
     }
     else
     {
-        hipLaunchKernelGGL((skipln_interleaved_kernel<G, false>), grid, dim3(kBlock), 0, stream, total, in, skip, beta,
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, false>), grid, block, dynLds, stream, total, in, skip, beta,
             gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
     }
     return check_launch("skipln_interleaved_kernel");
@@ -580,27 +584,35 @@ int skipln_interleaved(hipStream_t stream, bool large, bool mtron, int32_t ld, i
     float const eps = large ? 1.1920928955078125e-07f : 0.0009765625f;
     float const pmin = large ? -128.f : -127.f;
     int8_t* pre = mtron ? preln : nullptr;
+    // wavefronts per 8-token group: enough that every lane keeps at most 8 x 16 bytes per tensor, and
+    // small work units so that the loads of one workgroup overlap the arithmetic of another
+    static int const tune = [] {
+        char const* e = getenv("TRTAMD_SKIPLN_W");
+        return e ? atoi(e) : 0;
+    }();
+#define TRTAMD_IL(G, W, TOK)                                                                                          \
+    return launch_interleaved<G, W, TOK>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale,         \
+        qSkipScale, eps, pmin)
     switch (ld)
     {
     case 768:
-        return launch_interleaved<24>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
-            eps, pmin);
+        if (tune == 1) { TRTAMD_IL(24, 3, 8); }
+        if (tune == 2) { TRTAMD_IL(24, 3, 16); }
+        if (tune == 3) { TRTAMD_IL(24, 3, 32); }
+        TRTAMD_IL(24, 6, 32);
     case 1024:
-        return launch_interleaved<32>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
-            eps, pmin);
-    case 1536:
-        return launch_interleaved<48>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
-            eps, pmin);
-    case 2048:
-        return launch_interleaved<64>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
-            eps, pmin);
-    case 3072:
-        return launch_interleaved<96>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale, qSkipScale,
-            eps, pmin);
-    default:
-        return launch_interleaved<128>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale,
-            qSkipScale, eps, pmin);
+        if (tune == 1) { TRTAMD_IL(32, 2, 8); }
+        if (tune == 2) { TRTAMD_IL(32, 4, 16); }
+        if (tune == 3) { TRTAMD_IL(32, 4, 32); }
+        if (tune == 4) { TRTAMD_IL(32, 2, 16); }
+        if (tune == 5) { TRTAMD_IL(32, 16, 32); }
+        TRTAMD_IL(32, 8, 32);
+    case 1536: TRTAMD_IL(48, 8, 32);
+    case 2048: TRTAMD_IL(64, 8, 32);
+    case 3072: TRTAMD_IL(96, 16, 32);
+    default: TRTAMD_IL(128, 16, 32);
     }
+#undef TRTAMD_IL
 }
 
 } // namespace
