@@ -47,6 +47,13 @@ typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 
+// a * b rounded to binary32 on its own: the caller's following add must not absorb it into an fma
+__device__ inline float mul_rounded(float a, float b)
+{
+#pragma clang fp contract(off)
+    return a * b;
+}
+
 struct FmhaArgs
 {
     void const* qkv;
@@ -594,6 +601,320 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
 }
 
 // ------------------------------------------------------------------------------------------
+// INT8, prefix-valid keys (cu_seqlens or no mask at all): the usual case, specialised on the exact
+// number of 64-key blocks so that a query tile is one straight-line instruction stream.
+// ------------------------------------------------------------------------------------------
+
+// Stage K and V of one (sequence, head): rows < nk from memory, the rest of the last block zero.
+template <int KT, bool INTERLEAVED>
+__device__ inline void stage_kv_prefix_i8(FmhaArgs const& a, int64_t seqBase, int64_t firstTok, int n, int nk, int nkb,
+    uint8_t* sK, uint8_t* sV)
+{
+    constexpr int kRowsPerPass = kWavesI8 * kWaveSize / 4;   // 4 chunks of 16 bytes per 64-byte row
+    constexpr int kPasses = 64 / kRowsPerPass;
+    constexpr int kRow = Lds<1>::kRow;
+    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
+    int const chunk = threadIdx.x & 3;
+    int const rowInPass = threadIdx.x >> 2;
+    u32x4 kv[KT][kPasses], vv[KT][kPasses];
+#pragma unroll
+    for (int kb = 0; kb < KT; ++kb)
+    {
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p)
+        {
+            int const key = kb * 64 + p * kRowsPerPass + rowInPass;
+            kv[kb][p] = u32x4{0, 0, 0, 0};
+            vv[kb][p] = u32x4{0, 0, 0, 0};
+            if (key < nk)
+            {
+                kv[kb][p] = *reinterpret_cast<u32x4 const*>(
+                    src + qkv_chunk_offset<1, INTERLEAVED>(a, seqBase, firstTok, key, n, 1, chunk));
+                vv[kb][p] = *reinterpret_cast<u32x4 const*>(
+                    src + qkv_chunk_offset<1, INTERLEAVED>(a, seqBase, firstTok, key, n, 2, chunk));
+            }
+        }
+    }
+#pragma unroll
+    for (int kb = 0; kb < KT; ++kb)
+    {
+        if (kb < nkb)
+        {
+#pragma unroll
+            for (int p = 0; p < kPasses; ++p)
+            {
+                int const kk = p * kRowsPerPass + rowInPass;
+                int const kr = kb * 64 + kk;
+                int const vr = kb * 64 + v_row<1>(kk);
+                *reinterpret_cast<u32x4*>(sK + kr * kRow + swz<1>(kr, chunk) * 16) = kv[kb][p];
+                *reinterpret_cast<u32x4*>(sV + vr * kRow + swz<1>(vr, chunk) * 16) = vv[kb][p];
+            }
+        }
+    }
+}
+
+// All query tiles of this wavefront for a sequence of exactly NKB key blocks (the last one ragged).
+template <int NKB, bool INTERLEAVED, bool DEBUG>
+__device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, int const b, int const n,
+    int const part, uint8_t const* sK, uint8_t const* sV)
+{
+    constexpr int kRow = Lds<1>::kRow;
+    constexpr int NT = NKB * 4;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const wave = threadIdx.x >> 6;
+    int const lq = lane & 15;
+    int const g = lane >> 4;
+    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
+    int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
+
+    // last block: keys 64(NKB-1) + 16u + 4g + j exist for (16u + 4g + j) < lastKeys
+    int const lastKeys = sq.nk - (NKB - 1) * 64;
+    int const lastTiles = (lastKeys + 15) >> 4;
+    i32x4 const seedFull = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
+    int const lastRel = lastKeys - 4 * g; // key 16u + j of this lane group exists iff 16u + j < lastRel
+
+    auto load_q = [&](int qt) -> i32x4 {
+        int const qq = qt * kQPerWave + lq;
+        i32x4 v = {0, 0, 0, 0};
+        if (qq < sq.nq)
+        {
+            v = *reinterpret_cast<i32x4 const*>(
+                src + qkv_chunk_offset<1, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, g));
+        }
+        return v;
+    };
+    int const qtStep = a.qSplit * kWavesI8;
+    i32x4 qnext = load_q(part * kWavesI8 + wave);
+    for (int qt = part * kWavesI8 + wave; qt < nqt; qt += qtStep)
+    {
+        int const q = qt * kQPerWave + lq;
+        bool const qValid = q < sq.nq;
+        i32x4 const qreg = qnext;
+        qnext = load_q(qt + qtStep);
+
+        // ---- S^T = K Q^T; the int32 result reads as binary32 12582912 + acc, -inf for absent keys
+        i32x4 acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+        {
+            int const key = t * 16 + lq;
+            i32x4 const kreg = *reinterpret_cast<i32x4 const*>(sK + key * kRow + swz<1>(key, g) * 16);
+            i32x4 seed = seedFull;
+            if (t >= NT - 4)
+            {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    seed[j] = (16 * (t & 3) + j) < lastRel ? kMagicBits : kNegInfBits;
+                }
+            }
+            acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kreg, qreg, seed, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        if (DEBUG && a.dbgAcc1 && qValid)
+        {
+            for (int t = 0; t < NT; ++t)
+            {
+                for (int j = 0; j < 4; ++j)
+                {
+                    int const key = t * 16 + g * 4 + j;
+                    if (key < sq.nk)
+                    {
+                        a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key] = acc[t][j] - kMagicBits;
+                    }
+                }
+            }
+        }
+
+        // ---- row max on the biased integers (monotone in the score; -inf is a negative pattern)
+        int mx = kNegInfBits;
+#pragma unroll
+        for (int t = 0; t < NT; t += 2)
+        {
+            int const m0 = max(max(acc[t][0], acc[t][1]), max(acc[t][2], acc[t][3]));
+            int const m1 = max(max(acc[t + 1][0], acc[t + 1][1]), max(acc[t + 1][2], acc[t + 1][3]));
+            mx = max(mx, max(m0, m1));
+        }
+        mx = max(mx, __shfl_xor(mx, 16, kWaveSize));
+        mx = max(mx, __shfl_xor(mx, 32, kWaveSize));
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- e = 2^((acc - max) * c) in place, row sum
+        float const negK0 = -__int_as_float(mx) * a.c;
+        float sum0 = 0.f, sum1 = 0.f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+        {
+            if ((t & 3) == 0)
+            {
+                __builtin_amdgcn_sched_barrier(0); // bound the live temporaries to one key block
+            }
+            if (t >= NT - 4 && (t & 3) >= lastTiles)
+            {
+                continue; // tile without keys: its accumulators keep the -inf pattern (p8 = 0 below)
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                float const ev = __builtin_amdgcn_exp2f(fmaf(__int_as_float(acc[t][j]), a.c, negK0));
+                acc[t][j] = __float_as_int(ev);
+                if (j & 1)
+                {
+                    sum1 += ev;
+                }
+                else
+                {
+                    sum0 += ev;
+                }
+            }
+        }
+        float sum = sum0 + sum1;
+        sum += __shfl_xor(sum, 16, kWaveSize);
+        sum += __shfl_xor(sum, 32, kWaveSize);
+        float const r = a.scaleSoftmax / sum;   // sum >= 1: the row maximum contributes 2^0
+
+        // ---- p8 = rne(e * r), four keys to a dword; O^T = V^T P^T
+        i32x4 oacc[4];
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+        {
+            oacc[dt] = i32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+        {
+            __builtin_amdgcn_sched_barrier(0);
+            i32x4 preg = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                if (kb == NKB - 1 && u >= lastTiles)
+                {
+                    continue;
+                }
+                uint32_t yb[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    yb[j] = __float_as_uint(fmaf(__int_as_float(acc[kb * 4 + u][j]), r, kMagic));
+                }
+                uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+                uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+                preg[u] = (int) __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            }
+            if (DEBUG && a.dbgP8 && qValid)
+            {
+                for (int u = 0; u < 4; ++u)
+                {
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        int const key = kb * 64 + u * 16 + g * 4 + j;
+                        if (key < sq.nk)
+                        {
+                            a.dbgP8[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
+                                = (int8_t) ((uint32_t) preg[u] >> (8 * j));
+                        }
+                    }
+                }
+            }
+            int const vrow = kb * 64 + 8 * g + (lq >> 1);
+            uint8_t const* vbase = sV + vrow * kRow + 8 * (lq & 1);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+            {
+                int const sc = swz<1>(vrow, dt) * 16;
+                i32x2 const v0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + sc));
+                i32x2 const v1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + 32 * kRow + sc));
+                i32x4 const vreg = {v0[0], v0[1], v1[0], v1[1]};
+                oacc[dt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vreg, preg, oacc[dt], 0, 0, 0);
+            }
+        }
+
+        // ---- out8 = sat8(rne(acc2 * scale_bmm2)): binary32 product (rounded on its own, not fused
+        //      into the add), rounded to an integer through the magic constant, clamped on the bit
+        //      patterns (monotone for the positive results; anything negative is below the range)
+        if (qValid)
+        {
+            uint8_t* dst = static_cast<uint8_t*>(a.out);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+            {
+                uint32_t yb[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    int const bits = __float_as_int(mul_rounded((float) oacc[dt][j], a.scaleBmm2) + kMagic);
+                    yb[j] = (uint32_t) min(max(bits, kMagicBits - 128), kMagicBits + 127);
+                }
+                uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+                uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+                uint32_t const packed = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                int const d0 = dt * 16 + g * 4;
+                int64_t off;
+                if (INTERLEAVED)
+                {
+                    off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
+                }
+                else
+                {
+                    off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
+                }
+                *reinterpret_cast<uint32_t*>(dst + off) = packed;
+            }
+        }
+    }
+}
+
+template <int KT, bool INTERLEAVED, bool DEBUG>
+__global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_per_eu(KT <= 6 ? 3 : 2))) void fmha_i8_prefix_kernel(FmhaArgs const a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* sK = smem;
+    uint8_t* sV = smem + Lds<1>::matBytes(KT);
+    __shared__ int sLens[kMaxRanked + 1];
+    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
+    int const part = bid % a.qSplit;
+    int const n = (bid / a.qSplit) % a.N;
+    int const b = pick_sequence<kWavesI8 * kWaveSize>(a, bid / (a.qSplit * a.N), sLens);
+    SeqInfo const sq = seq_info(a, b, KT * 64);
+    int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
+    if (part * kWavesI8 >= nqt)
+    {
+        return; // no query tile for this workgroup (also: empty sequence)
+    }
+    int const nkb = (sq.nk + 63) >> 6;
+    stage_kv_prefix_i8<KT, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sK, sV);
+    __syncthreads();
+    switch (nkb)
+    {
+    case 1: attend_i8<1, INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV); break;
+    case 2:
+        if (KT >= 2) attend_i8<(KT >= 2 ? 2 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    case 3:
+        if (KT >= 3) attend_i8<(KT >= 3 ? 3 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    case 4:
+        if (KT >= 4) attend_i8<(KT >= 4 ? 4 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    case 5:
+        if (KT >= 5) attend_i8<(KT >= 5 ? 5 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    case 6:
+        if (KT >= 6) attend_i8<(KT >= 6 ? 6 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    case 7:
+        if (KT >= 7) attend_i8<(KT >= 7 ? 7 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    case 8:
+        if (KT >= 8) attend_i8<(KT >= 8 ? 8 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        break;
+    default: break;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // FP16
 // ------------------------------------------------------------------------------------------
 template <int KT, bool DEBUG>
@@ -864,6 +1185,32 @@ template <bool DEBUG>
 int run_i8(hipStream_t stream, FmhaArgs const& a, bool interleaved)
 {
     int const kt = pick_kt(a.S);
+    // keys are a valid prefix (cu_seqlens, or no mask) and probabilities cannot leave the INT8 range:
+    // the kernel specialised on the number of key blocks serves the launch
+    static int const noFast = [] {
+        char const* e = getenv("TRTAMD_FMHA_GENERIC");
+        return e ? atoi(e) : 0;
+    }();
+    if (a.packedMask == nullptr && !a.clampP && !noFast)
+    {
+#define TRTAMD_I8P(KT)                                                                                                 \
+    case KT:                                                                                                           \
+        return interleaved ? launch_fmha(fmha_i8_prefix_kernel<KT, true, DEBUG>, "fmha_i8_prefix_interleaved", stream, \
+                   a, Lds<1>::total(KT), kWavesI8)                                                                     \
+                           : launch_fmha(fmha_i8_prefix_kernel<KT, false, DEBUG>, "fmha_i8_prefix", stream, a,         \
+                               Lds<1>::total(KT), kWavesI8)
+        switch (kt)
+        {
+            TRTAMD_I8P(1);
+            TRTAMD_I8P(2);
+            TRTAMD_I8P(3);
+            TRTAMD_I8P(4);
+            TRTAMD_I8P(6);
+            TRTAMD_I8P(8);
+        default: break;
+        }
+#undef TRTAMD_I8P
+    }
 #define TRTAMD_I8(KT)                                                                                                  \
     case KT:                                                                                                           \
         return interleaved ? launch_fmha(fmha_i8_kernel<KT, true, DEBUG>, "fmha_i8_interleaved", stream, a,           \
