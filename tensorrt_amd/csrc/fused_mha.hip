@@ -600,6 +600,86 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
     }
 }
 
+// Sequence selection for the var-seqlen kernels with a single trip to global memory: all B+1
+// cu_seqlens values go to LDS, sequences are ordered longest first by 16-token bucket (ties by
+// index) with a histogram, and the workgroup looks up the sequence at its own position.  Every
+// workgroup computes the same order, so no state outside the launch is needed.
+constexpr int kLenBuckets = 34; // (length + 15) / 16 for lengths 0 .. 512, and one for longer
+struct PickLds
+{
+    int cu[kMaxRanked + 1];
+    int hist[kLenBuckets];
+};
+
+__device__ inline int len_bucket(int len)
+{
+    return min(max(len + 15, 0) >> 4, kLenBuckets - 1);
+}
+
+template <int THREADS>
+__device__ inline SeqInfo pick_sequence_info(FmhaArgs const& a, int rank, int capacity, PickLds& l, int& bOut)
+{
+    if (a.cuSeqlens == nullptr || a.B > kMaxRanked)
+    {
+        bOut = rank; // fixed layout (equal lengths) or too many sequences: natural order
+        return seq_info(a, rank, capacity);
+    }
+    if (threadIdx.x < kLenBuckets)
+    {
+        l.hist[threadIdx.x] = 0;
+    }
+    for (int t = threadIdx.x; t <= a.B; t += THREADS)
+    {
+        l.cu[t] = a.cuSeqlens[t];
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < a.B; t += THREADS)
+    {
+        atomicAdd(&l.hist[len_bucket(l.cu[t + 1] - l.cu[t])], 1);
+    }
+    __syncthreads();
+    // bucket that holds position `rank` (longest bucket first) and the offset inside it
+    int k = kLenBuckets - 1;
+    int off = rank;
+    for (; k > 0; --k)
+    {
+        int const c = l.hist[k];
+        if (off < c)
+        {
+            break;
+        }
+        off -= c;
+    }
+    // the off-th sequence (by index) of bucket k: every wavefront scans on its own
+    int b = a.B - 1;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    for (int t0 = 0; t0 < a.B; t0 += kWaveSize)
+    {
+        int const t = t0 + lane;
+        bool const in = t < a.B && len_bucket(l.cu[t + 1] - l.cu[t]) == k;
+        uint64_t const m = __ballot(in);
+        int const c = __popcll(m);
+        if (off < c)
+        {
+            int const before = __popcll(m & ((1ull << lane) - 1ull));
+            uint64_t const hit = __ballot(in && before == off);
+            b = t0 + (int) __builtin_ctzll(hit);
+            break;
+        }
+        off -= c;
+    }
+    bOut = b;
+    SeqInfo s;
+    int const first = l.cu[b];
+    int const len = min(max(l.cu[b + 1] - first, 0), capacity);
+    s.firstTok = first;
+    s.seqBaseIn = (int64_t) first * a.tokStrideIn;
+    s.seqBaseOut = (int64_t) first * a.tokStrideOut;
+    s.nq = len;
+    s.nk = len;
+    return s;
+}
+
 // ------------------------------------------------------------------------------------------
 // INT8, prefix-valid keys (cu_seqlens or no mask at all): the usual case, specialised on the exact
 // number of 64-key blocks so that a query tile is one straight-line instruction stream.
@@ -656,7 +736,7 @@ __device__ inline void stage_kv_prefix_i8(FmhaArgs const& a, int64_t seqBase, in
 // All query tiles of this wavefront for a sequence of exactly NKB key blocks (the last one ragged).
 template <int NKB, bool INTERLEAVED, bool DEBUG>
 __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, int const b, int const n,
-    int const part, uint8_t const* sK, uint8_t const* sV)
+    int const qtBegin, int const qtEnd, uint8_t const* sK, uint8_t const* sV, i32x4 const qFirst)
 {
     constexpr int kRow = Lds<1>::kRow;
     constexpr int NT = NKB * 4;
@@ -665,7 +745,6 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
     int const lq = lane & 15;
     int const g = lane >> 4;
     uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
-    int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
 
     // last block: keys 64(NKB-1) + 16u + 4g + j exist for (16u + 4g + j) < lastKeys
     int const lastKeys = sq.nk - (NKB - 1) * 64;
@@ -683,9 +762,9 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
         }
         return v;
     };
-    int const qtStep = a.qSplit * kWavesI8;
-    i32x4 qnext = load_q(part * kWavesI8 + wave);
-    for (int qt = part * kWavesI8 + wave; qt < nqt; qt += qtStep)
+    constexpr int qtStep = kWavesI8;
+    i32x4 qnext = qFirst; // requested by the caller together with K and V
+    for (int qt = qtBegin + wave; qt < qtEnd; qt += qtStep)
     {
         int const q = qt * kQPerWave + lq;
         bool const qValid = q < sq.nq;
@@ -728,14 +807,15 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
         }
 
         // ---- row max on the biased integers (monotone in the score; -inf is a negative pattern)
-        int mx = kNegInfBits;
+        // two chains of three-input maxima (v_max3_i32): one instruction per two scores
+        int mxA = kNegInfBits, mxB = kNegInfBits;
 #pragma unroll
-        for (int t = 0; t < NT; t += 2)
+        for (int t = 0; t < NT; ++t)
         {
-            int const m0 = max(max(acc[t][0], acc[t][1]), max(acc[t][2], acc[t][3]));
-            int const m1 = max(max(acc[t + 1][0], acc[t + 1][1]), max(acc[t + 1][2], acc[t + 1][3]));
-            mx = max(mx, max(m0, m1));
+            mxA = max(max(mxA, acc[t][0]), acc[t][1]);
+            mxB = max(max(mxB, acc[t][2]), acc[t][3]);
         }
+        int mx = max(mxA, mxB);
         mx = max(mx, __shfl_xor(mx, 16, kWaveSize));
         mx = max(mx, __shfl_xor(mx, 32, kWaveSize));
         __builtin_amdgcn_sched_barrier(0);
@@ -872,43 +952,57 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* sK = smem;
     uint8_t* sV = smem + Lds<1>::matBytes(KT);
-    __shared__ int sLens[kMaxRanked + 1];
+    __shared__ PickLds sPick;
     uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
     int const part = bid % a.qSplit;
     int const n = (bid / a.qSplit) % a.N;
-    int const b = pick_sequence<kWavesI8 * kWaveSize>(a, bid / (a.qSplit * a.N), sLens);
-    SeqInfo const sq = seq_info(a, b, KT * 64);
+    int b;
+    SeqInfo const sq = pick_sequence_info<kWavesI8 * kWaveSize>(a, bid / (a.qSplit * a.N), KT * 64, sPick, b);
+    // contiguous tile ranges, each a multiple of one round of the workgroup's wavefronts
     int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
-    if (part * kWavesI8 >= nqt)
+    int const per = kWavesI8 * ((nqt + kWavesI8 * a.qSplit - 1) / (kWavesI8 * a.qSplit));
+    int const qtBegin = min(part * per, nqt);
+    int const qtEnd = min(qtBegin + per, nqt);
+    if (qtBegin >= qtEnd)
     {
         return; // no query tile for this workgroup (also: empty sequence)
     }
     int const nkb = (sq.nk + 63) >> 6;
+    // the first query tile of this wavefront travels with K and V
+    i32x4 qFirst = {0, 0, 0, 0};
+    {
+        int const qq = (qtBegin + (int) (threadIdx.x >> 6)) * kQPerWave + (int) (threadIdx.x & 15);
+        if (qq < sq.nq && qtBegin + (int) (threadIdx.x >> 6) < qtEnd)
+        {
+            qFirst = *reinterpret_cast<i32x4 const*>(static_cast<uint8_t const*>(a.qkv)
+                + qkv_chunk_offset<1, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, (threadIdx.x & 63) >> 4));
+        }
+    }
     stage_kv_prefix_i8<KT, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sK, sV);
     __syncthreads();
     switch (nkb)
     {
-    case 1: attend_i8<1, INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV); break;
+    case 1: attend_i8<1, INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst); break;
     case 2:
-        if (KT >= 2) attend_i8<(KT >= 2 ? 2 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 2) attend_i8<(KT >= 2 ? 2 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     case 3:
-        if (KT >= 3) attend_i8<(KT >= 3 ? 3 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 3) attend_i8<(KT >= 3 ? 3 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     case 4:
-        if (KT >= 4) attend_i8<(KT >= 4 ? 4 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 4) attend_i8<(KT >= 4 ? 4 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     case 5:
-        if (KT >= 5) attend_i8<(KT >= 5 ? 5 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 5) attend_i8<(KT >= 5 ? 5 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     case 6:
-        if (KT >= 6) attend_i8<(KT >= 6 ? 6 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 6) attend_i8<(KT >= 6 ? 6 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     case 7:
-        if (KT >= 7) attend_i8<(KT >= 7 ? 7 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 7) attend_i8<(KT >= 7 ? 7 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     case 8:
-        if (KT >= 8) attend_i8<(KT >= 8 ? 8 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, part, sK, sV);
+        if (KT >= 8) attend_i8<(KT >= 8 ? 8 : 1), INTERLEAVED, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst);
         break;
     default: break;
     }
