@@ -1229,6 +1229,296 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
 }
 
 // ------------------------------------------------------------------------------------------
+// FP16, prefix-valid keys: same specialisation on the number of 64-key blocks as the INT8 kernel.
+// ------------------------------------------------------------------------------------------
+
+template <int KT>
+__device__ inline void stage_kv_prefix_f16(FmhaArgs const& a, int64_t seqBase, int64_t firstTok, int n, int nk,
+    int nkb, uint8_t* sK, uint8_t* sV)
+{
+    constexpr int kRowsPerPass = kWavesF16 * kWaveSize / 8;   // 8 chunks of 16 bytes per 128-byte row
+    constexpr int kPasses = 64 / kRowsPerPass;
+    constexpr int kRow = Lds<2>::kRow;
+    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
+    int const chunk = threadIdx.x & 7;
+    int const rowInPass = threadIdx.x >> 3;
+    u32x4 kv[KT][kPasses], vv[KT][kPasses];
+#pragma unroll
+    for (int kb = 0; kb < KT; ++kb)
+    {
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p)
+        {
+            int const key = kb * 64 + p * kRowsPerPass + rowInPass;
+            kv[kb][p] = u32x4{0, 0, 0, 0};
+            vv[kb][p] = u32x4{0, 0, 0, 0};
+            if (key < nk)
+            {
+                kv[kb][p] = *reinterpret_cast<u32x4 const*>(
+                    src + qkv_chunk_offset<2, false>(a, seqBase, firstTok, key, n, 1, chunk));
+                vv[kb][p] = *reinterpret_cast<u32x4 const*>(
+                    src + qkv_chunk_offset<2, false>(a, seqBase, firstTok, key, n, 2, chunk));
+            }
+        }
+    }
+#pragma unroll
+    for (int kb = 0; kb < KT; ++kb)
+    {
+        if (kb < nkb)
+        {
+#pragma unroll
+            for (int p = 0; p < kPasses; ++p)
+            {
+                int const kk = p * kRowsPerPass + rowInPass;
+                int const kr = kb * 64 + kk;
+                int const vr = kb * 64 + v_row<2>(kk);
+                *reinterpret_cast<u32x4*>(sK + kr * kRow + swz<2>(kr, chunk) * 16) = kv[kb][p];
+                *reinterpret_cast<u32x4*>(sV + vr * kRow + swz<2>(vr, chunk) * 16) = vv[kb][p];
+            }
+        }
+    }
+}
+
+template <int NKB, bool DEBUG>
+__device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq, int const b, int const n,
+    int const qtBegin, int const qtEnd, uint8_t const* sK, uint8_t const* sV, f16x8 const qFirst0,
+    f16x8 const qFirst1)
+{
+    constexpr int kRow = Lds<2>::kRow;
+    constexpr int NT = NKB * 4;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const wave = threadIdx.x >> 6;
+    int const lq = lane & 15;
+    int const g = lane >> 4;
+    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
+    f16x8 ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+    {
+        ones[i] = (f16) 1.f;
+    }
+    int const lastKeys = sq.nk - (NKB - 1) * 64;
+    int const lastHalves = (lastKeys + 31) >> 5;   // 32-key halves of the last block that hold keys
+    int const lastRel = lastKeys - 4 * g;          // key 16u + j of this lane group exists iff 16u + j < lastRel
+
+    auto load_q = [&](int qt, int h) -> f16x8 {
+        int const qq = qt * kQPerWave + lq;
+        u32x4 raw = {0, 0, 0, 0};
+        if (qq < sq.nq)
+        {
+            raw = *reinterpret_cast<u32x4 const*>(
+                src + qkv_chunk_offset<2, false>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, h * 4 + g));
+        }
+        return __builtin_bit_cast(f16x8, raw);
+    };
+    f16x8 qnext[2] = {qFirst0, qFirst1};
+    for (int qt = qtBegin + wave; qt < qtEnd; qt += kWavesF16)
+    {
+        int const q = qt * kQPerWave + lq;
+        bool const qValid = q < sq.nq;
+        f16x8 const qreg[2] = {qnext[0], qnext[1]};
+        qnext[0] = load_q(qt + kWavesF16, 0);
+        qnext[1] = load_q(qt + kWavesF16, 1);
+
+        // ---- S^T = K Q^T (binary32 accumulation); absent keys start from -infinity
+        f32x4 acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+        {
+            int const key = t * 16 + lq;
+            f32x4 sd = {0.f, 0.f, 0.f, 0.f};
+            if (t >= NT - 4)
+            {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    sd[j] = (16 * (t & 3) + j) < lastRel ? 0.f : -__builtin_inff();
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+            {
+                f16x8 const kreg = *reinterpret_cast<f16x8 const*>(sK + key * kRow + swz<2>(key, h * 4 + g) * 16);
+                sd = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg, qreg[h], sd, 0, 0, 0);
+            }
+            acc[t] = sd;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        if (DEBUG && a.dbgAcc1 && qValid)
+        {
+            for (int t = 0; t < NT; ++t)
+            {
+                for (int j = 0; j < 4; ++j)
+                {
+                    int const key = t * 16 + g * 4 + j;
+                    if (key < sq.nk)
+                    {
+                        a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key] = __float_as_int(acc[t][j]);
+                    }
+                }
+            }
+        }
+
+        // ---- row max
+        float mxA = -__builtin_inff(), mxB = -__builtin_inff();
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+        {
+            mxA = fmaxf(fmaxf(mxA, acc[t][0]), acc[t][1]);
+            mxB = fmaxf(fmaxf(mxB, acc[t][2]), acc[t][3]);
+        }
+        float mx = fmaxf(mxA, mxB);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, kWaveSize));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWaveSize));
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- p = 2^((s - max) * c) rounded to binary16; O^T = V^T P^T; row sum by a tile of ones
+        float const negK0 = -mx * a.c; // nk >= 1: the maximum is finite
+        f32x4 oacc[4];
+        f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+        {
+            oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+        {
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb)
+            {
+                if (kb == NKB - 1 && hb >= lastHalves)
+                {
+                    continue; // no key in this half
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                f16x8 preg;
+#pragma unroll
+                for (int w = 0; w < 2; ++w)
+                {
+                    int const t = kb * 4 + hb * 2 + w;
+                    float pr[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        pr[j] = __builtin_amdgcn_exp2f(fmaf(acc[t][j], a.c, negK0));
+                    }
+                    f16x2 const p01 = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(pr[0], pr[1]));
+                    f16x2 const p23 = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(pr[2], pr[3]));
+                    preg[w * 4 + 0] = p01[0];
+                    preg[w * 4 + 1] = p01[1];
+                    preg[w * 4 + 2] = p23[0];
+                    preg[w * 4 + 3] = p23[1];
+                }
+                int const vrow = kb * 64 + hb * 32 + 4 * g + (lq >> 2);
+                uint8_t const* vbase = sV + vrow * kRow + 8 * (lq & 1);
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+                {
+                    int const sc = swz<2>(vrow, 2 * dt + ((lq >> 1) & 1)) * 16;
+                    i16x4 const v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vbase + sc));
+                    i16x4 const v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vbase + 16 * kRow + sc));
+                    typedef short i16x8 __attribute__((ext_vector_type(8)));
+                    i16x8 const both = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(f16x8, both), preg, oacc[dt], 0, 0, 0);
+                }
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, preg, sacc, 0, 0, 0);
+            }
+        }
+
+        if (qValid)
+        {
+            float const rinv = 1.f / sacc[0];
+            uint8_t* dst = static_cast<uint8_t*>(a.out);
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+            {
+                f16x4 y;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    y[j] = (f16) (oacc[dt][j] * rinv);
+                }
+                int const d0 = dt * 16 + g * 4;
+                int64_t const off
+                    = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + d0) * 2;
+                *reinterpret_cast<u32x2*>(dst + off) = __builtin_bit_cast(u32x2, y);
+            }
+        }
+    }
+}
+
+template <int KT, bool DEBUG>
+__global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_prefix_kernel(FmhaArgs const a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* sK = smem;
+    uint8_t* sV = smem + Lds<2>::matBytes(KT);
+    __shared__ PickLds sPick;
+    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
+    int const part = bid % a.qSplit;
+    int const n = (bid / a.qSplit) % a.N;
+    int b;
+    SeqInfo const sq = pick_sequence_info<kWavesF16 * kWaveSize>(a, bid / (a.qSplit * a.N), KT * 64, sPick, b);
+    int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
+    int const per = kWavesF16 * ((nqt + kWavesF16 * a.qSplit - 1) / (kWavesF16 * a.qSplit));
+    int const qtBegin = min(part * per, nqt);
+    int const qtEnd = min(qtBegin + per, nqt);
+    if (qtBegin >= qtEnd)
+    {
+        return;
+    }
+    int const nkb = (sq.nk + 63) >> 6;
+    f16x8 qFirst[2];
+    {
+        int const qt = qtBegin + (int) (threadIdx.x >> 6);
+        int const qq = qt * kQPerWave + (int) (threadIdx.x & 15);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+        {
+            u32x4 raw = {0, 0, 0, 0};
+            if (qq < sq.nq && qt < qtEnd)
+            {
+                raw = *reinterpret_cast<u32x4 const*>(static_cast<uint8_t const*>(a.qkv)
+                    + qkv_chunk_offset<2, false>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0,
+                        h * 4 + (int) ((threadIdx.x & 63) >> 4)));
+            }
+            qFirst[h] = __builtin_bit_cast(f16x8, raw);
+        }
+    }
+    stage_kv_prefix_f16<KT>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sK, sV);
+    __syncthreads();
+    switch (nkb)
+    {
+    case 1: attend_f16<1, DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]); break;
+    case 2:
+        if (KT >= 2) attend_f16<(KT >= 2 ? 2 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    case 3:
+        if (KT >= 3) attend_f16<(KT >= 3 ? 3 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    case 4:
+        if (KT >= 4) attend_f16<(KT >= 4 ? 4 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    case 5:
+        if (KT >= 5) attend_f16<(KT >= 5 ? 5 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    case 6:
+        if (KT >= 6) attend_f16<(KT >= 6 ? 6 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    case 7:
+        if (KT >= 7) attend_f16<(KT >= 7 ? 7 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    case 8:
+        if (KT >= 8) attend_f16<(KT >= 8 ? 8 : 1), DEBUG>(a, sq, b, n, qtBegin, qtEnd, sK, sV, qFirst[0], qFirst[1]);
+        break;
+    default: break;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 
@@ -1329,6 +1619,27 @@ template <bool DEBUG>
 int run_f16(hipStream_t stream, FmhaArgs const& a)
 {
     int const kt = pick_kt(a.S);
+    static int const noFast = [] {
+        char const* e = getenv("TRTAMD_FMHA_GENERIC");
+        return e ? atoi(e) : 0;
+    }();
+    if (a.packedMask == nullptr && !noFast)
+    {
+#define TRTAMD_F16P(KT)                                                                                                \
+    case KT:                                                                                                           \
+        return launch_fmha(fmha_f16_prefix_kernel<KT, DEBUG>, "fmha_f16_prefix", stream, a, Lds<2>::total(KT), kWavesF16)
+        switch (kt)
+        {
+            TRTAMD_F16P(1);
+            TRTAMD_F16P(2);
+            TRTAMD_F16P(3);
+            TRTAMD_F16P(4);
+            TRTAMD_F16P(6);
+            TRTAMD_F16P(8);
+        default: break;
+        }
+#undef TRTAMD_F16P
+    }
 #define TRTAMD_F16(KT)                                                                                                 \
     case KT: return launch_fmha(fmha_f16_kernel<KT, DEBUG>, "fmha_f16", stream, a, Lds<2>::total(KT), kWavesF16)
     switch (kt)
@@ -1415,13 +1726,16 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
     a.N = p->h;
     a.S = p->s;
     {
-        // Workgroups per (sequence, head): one, unless the launch would leave compute units idle
-        // (fewer than ~4 workgroups per CU) and the rows are long enough to share.
+        // Workgroups per (sequence, head): one, unless the launch would leave compute units idle.
+        // Every extra workgroup stages K and V again, which costs more than it gains once the
+        // chip is full, so heads are only shared while there are fewer of them than workgroup slots
+        // worth filling (one per CU for FP16, whose K/V take most of a CU's LDS; two for INT8).
         int const waves = dataType == 2 ? kWavesI8 : kWavesF16;
         int const maxSplit = std::max(1, ceil_div(ceil_div(p->s, kQPerWave), waves));
         int64_t const heads = (int64_t) p->b * p->h;
+        int64_t const target = dataType == 2 ? 512 : 256;
         int split = 1;
-        while (split < maxSplit && heads * split < 1024)
+        while (split < maxSplit && heads * split < target)
         {
             split *= 2;
         }

@@ -262,8 +262,12 @@ int skip_layer_norm(hipStream_t stream, int32_t ld, int64_t n, T const* in, T co
 
 // ------------------------------------------------------------------------------------------
 // INT8 rows, linear layout (skiplnDQQ, skipLayerNormKernel.cu:43-106): each lane owns 16
-// consecutive channels of a row, a wave owns R rows.  v = dqIn*in + dqSkip*skip (+bias) in
-// binary32, Welford statistics, epsilon 2^-10, out = sat8(rne(y * qScale)).
+// consecutive channels of a row, a wave owns R rows.  v = dqIn*in + dqSkip*skip (+bias),
+// epsilon 2^-10, out = sat8(rne(y * qScale)).  The statistics are exact: integer dot products of
+// the bytes (v_dot4_i32_i8) summed over the wave, the bias terms as binary32 dot products, all
+// combined in binary64.  gamma*qScale and beta*qScale of the lane's 16 channels stay in registers
+// for all rows; bytes are converted through the unsigned path (x + 128) with the offset folded into
+// the additive constant, and rounded by the 1.5*2^23 constant.
 // ------------------------------------------------------------------------------------------
 template <int R, bool HAS_BIAS>
 __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_t const rows,
@@ -279,83 +283,128 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
         return;
     }
     bool const lane_ok = lane * 16 < ld;
+    int const ch = lane_ok ? lane * 16 : 0;
     u32x4 xi[R], xs[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)
     {
-        bool const ok = lane_ok && row0 + r < rows;
-        int64_t const off = (row0 + r) * ld + lane * 16;
-        xi[r] = ok ? *reinterpret_cast<u32x4 const*>(in + off) : u32x4{0, 0, 0, 0};
-        xs[r] = ok ? *reinterpret_cast<u32x4 const*>(skip + off) : u32x4{0, 0, 0, 0};
+        // rows past the end re-read the last row (and store nothing); idle lanes contribute zeros
+        int64_t const row = min(row0 + r, rows - 1);
+        int64_t const off = row * ld + ch;
+        xi[r] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(in + off));
+        xs[r] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(skip + off));
+        if (!lane_ok)
+        {
+            xi[r] = u32x4{0, 0, 0, 0};
+            xs[r] = u32x4{0, 0, 0, 0};
+        }
     }
-    Vec16<f16> g[2], b[2], bs[2];
+    float gq[16], bq[16], bs[16];
+    float biasSum = 0.f, biasSq = 0.f;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
     {
-        int const c = lane * 16 + h * 8;
-        g[h].u = lane_ok ? *reinterpret_cast<u32x4 const*>(gamma + c) : u32x4{0, 0, 0, 0};
-        b[h].u = lane_ok ? *reinterpret_cast<u32x4 const*>(beta + c) : u32x4{0, 0, 0, 0};
+        Vec16<f16> g, b, c;
+        g.u = *reinterpret_cast<u32x4 const*>(gamma + ch + h * 8);
+        b.u = *reinterpret_cast<u32x4 const*>(beta + ch + h * 8);
         if (HAS_BIAS)
         {
-            bs[h].u = lane_ok ? *reinterpret_cast<u32x4 const*>(bias + c) : u32x4{0, 0, 0, 0};
+            c.u = *reinterpret_cast<u32x4 const*>(bias + ch + h * 8);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+        {
+            gq[h * 8 + k] = (float) g.e[k] * qScale;
+            bq[h * 8 + k] = (float) b.e[k] * qScale;
+            if (HAS_BIAS)
+            {
+                float const v = lane_ok ? (float) c.e[k] : 0.f;
+                bs[h * 8 + k] = v;
+                biasSum += v;
+                biasSq += v * v;
+            }
         }
     }
-    float const rld = 1.f / (float) ld;
+    if (HAS_BIAS)
+    {
+        biasSum = wave_sum(biasSum);
+        biasSq = wave_sum(biasSq);
+    }
+    double const dIn = (double) dqIn, dSk = (double) dqSkip;
+    double const rld = 1.0 / (double) ld;
+    constexpr float kMagic = 12582912.f;
 #pragma unroll
     for (int r = 0; r < R; ++r)
     {
-        if (row0 + r >= rows)
-        {
-            break;
-        }
-        float v[16];
-        float sum = 0.f;
+        int sIn = 0, sSk = 0, sII = 0, sIS = 0, sSS = 0;
+        float dotIn = 0.f, dotSk = 0.f; // sum bias*in, sum bias*skip
 #pragma unroll
-        for (int k = 0; k < 16; ++k)
+        for (int q = 0; q < 4; ++q)
         {
-            float x = dqIn * i8_to_f32(xi[r][k >> 2], k & 3) + dqSkip * i8_to_f32(xs[r][k >> 2], k & 3);
+            sIn = __builtin_amdgcn_sdot4((int) xi[r][q], 0x01010101, sIn, false);
+            sSk = __builtin_amdgcn_sdot4((int) xs[r][q], 0x01010101, sSk, false);
+            sII = __builtin_amdgcn_sdot4((int) xi[r][q], (int) xi[r][q], sII, false);
+            sIS = __builtin_amdgcn_sdot4((int) xi[r][q], (int) xs[r][q], sIS, false);
+            sSS = __builtin_amdgcn_sdot4((int) xs[r][q], (int) xs[r][q], sSS, false);
             if (HAS_BIAS)
             {
-                x += (float) bs[k >> 3].e[k & 7];
-            }
-            v[k] = x;
-            sum += x;
-        }
-        Welford w;
-        w.n = lane_ok ? 16.f : 0.f;
-        w.mean = sum * (1.f / 16.f);
-        w.m2 = 0.f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k)
-        {
-            float const dlt = v[k] - w.mean;
-            w.m2 += dlt * dlt;
-        }
-        if (!lane_ok)
-        {
-            w.mean = 0.f;
-            w.m2 = 0.f;
-        }
-        w = group_welford<kWaveSize>(w);
-        float const mu = w.mean;
-        float const rsigma = rsqrtf(w.m2 * rld + 0.0009765625f);
-        if (lane_ok)
-        {
-            u32x4 o;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                int p[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
                 {
-                    int const c = q * 4 + k;
-                    float const y = (float) g[c >> 3].e[c & 7] * (v[c] - mu) * rsigma + (float) b[c >> 3].e[c & 7];
-                    p[k] = sat8_rne(y * qScale);
+                    dotIn = fmaf(i8_to_f32(xi[r][q], k), bs[q * 4 + k], dotIn);
+                    dotSk = fmaf(i8_to_f32(xs[r][q], k), bs[q * 4 + k], dotSk);
                 }
-                o[q] = pack_i8x4(p[0], p[1], p[2], p[3]);
             }
-            *reinterpret_cast<u32x4*>(out + (row0 + r) * ld + lane * 16) = o;
+        }
+#pragma unroll
+        for (int m = 1; m < kWaveSize; m *= 2)
+        {
+            sIn += __shfl_xor(sIn, m, kWaveSize);
+            sSk += __shfl_xor(sSk, m, kWaveSize);
+            sII += __shfl_xor(sII, m, kWaveSize);
+            sIS += __shfl_xor(sIS, m, kWaveSize);
+            sSS += __shfl_xor(sSS, m, kWaveSize);
+        }
+        double sum1 = dIn * sIn + dSk * sSk;
+        double sum2 = dIn * dIn * sII + 2.0 * dIn * dSk * sIS + dSk * dSk * sSS;
+        if (HAS_BIAS)
+        {
+            dotIn = wave_sum(dotIn);
+            dotSk = wave_sum(dotSk);
+            sum1 += (double) biasSum;
+            sum2 += 2.0 * (dIn * (double) dotIn + dSk * (double) dotSk) + (double) biasSq;
+        }
+        double const mean = sum1 * rld;
+        float const var = (float) (sum2 * rld - mean * mean);
+        float const rsigma = rsqrtf(fmaxf(var, 0.f) + 0.0009765625f);
+        float const a1 = dqIn * rsigma;
+        float const a2 = dqSkip * rsigma;
+        float const c1 = (float) ((-128.0 * (dIn + dSk) - mean) * (double) rsigma);
+        u32x4 o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            uint32_t const ua = xi[r][q] ^ 0x80808080u;
+            uint32_t const us = xs[r][q] ^ 0x80808080u;
+            uint32_t yb[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                float const fa = (float) ((ua >> (8 * k)) & 0xffu);
+                float const fs = (float) ((us >> (8 * k)) & 0xffu);
+                float const c = HAS_BIAS ? fmaf(bs[q * 4 + k], rsigma, c1) : c1;
+                float const nrm = fmaf(fa, a1, fmaf(fs, a2, c));
+                float y = fmaf(gq[q * 4 + k], nrm, bq[q * 4 + k]);
+                y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
+                yb[k] = __float_as_uint(y + kMagic);
+            }
+            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+            o[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+        if (lane_ok && row0 + r < rows)
+        {
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + (row0 + r) * ld + ch));
         }
     }
 }
