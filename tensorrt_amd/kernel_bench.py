@@ -104,6 +104,25 @@ def main():
                                                           biash.data_ptr())))
     report("SkipLN fp16 4096x768", t, nbytes=n_rows * ld * 3 * 2 + 3 * ld * 2)
 
+    # ---- the same kernels at a size where the launch itself no longer matters -------------------
+    n_big = 65536
+    xb = torch.randn((n_big, ld), dtype=torch.float16, device="cuda")
+    sb = torch.randn((n_big, ld), dtype=torch.float16, device="cuda")
+    ob = torch.empty_like(xb)
+    t = timeit(lambda: api.check(api.skip_layer_norm_fp16(stream, ld, n_big * ld, xb.data_ptr(), sb.data_ptr(),
+                                                          bh.data_ptr(), gh.data_ptr(), ob.data_ptr(),
+                                                          biash.data_ptr())))
+    report("SkipLN fp16 65536x768", t, nbytes=n_big * ld * 3 * 2 + 3 * ld * 2)
+    Sb, Bb = 384, 256
+    idsb = dev(r.integers(0, vocab, (Sb, Bb)).astype(np.int32))
+    segsb = dev(r.integers(0, 2, (Sb, Bb)).astype(np.int32))
+    embb = torch.empty((Sb * Bb, ld), dtype=torch.float16, device="cuda")
+    t = timeit(lambda: api.check(api.emb_layer_norm_fp16(stream, ld, Bb, Sb, idsb.data_ptr(), segsb.data_ptr(),
+                                                         b32.data_ptr(), g32.data_ptr(), word.data_ptr(),
+                                                         pos.data_ptr(), tok.data_ptr(), vocab, 2, embb.data_ptr())))
+    report("EmbLN fp16 B256 S384 E768", t, nbytes=Sb * Bb * (2 * ld * 2 + 8) + Sb * ld * 2 + 2 * ld * 2)
+    del xb, sb, ob, embb
+
     # ---- fused attention FP16, BERT-base, B=32, var-seqlen ---------------------------------------
     for S in (128, 384):
         B, N, d = 32, 12, 64
