@@ -24,35 +24,111 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kWaveSize = 64;
 
 // ---- wave64 reductions -------------------------------------------------------------------
+// All cross-lane steps stay in the vector ALU: DPP inside a row of 16 lanes, v_permlane16_swap /
+// v_permlane32_swap (gfx950) across rows.  ds_bpermute (what __shfl_xor compiles to) would send
+// every step through the LDS crossbar.
+
+template <typename To, typename From>
+__device__ inline To bits_as(From v)
+{
+    static_assert(sizeof(To) == sizeof(From), "same size");
+    return __builtin_bit_cast(To, v);
+}
+
+// One butterfly step: combines v with the value of a lane of the "other" M-lane group (the lane
+// index differs in bit log2(M); lower bits may differ too, which is immaterial once the lower steps
+// have been taken).  Steps must therefore be applied in the order M = 1, 2, 4, 8, 16, 32.
+template <int M, typename T, typename Op>
+__device__ inline T reduce_step(T v, Op op)
+{
+    static_assert(sizeof(T) == 4, "32-bit values");
+    int const bits = bits_as<int>(v);
+    if constexpr (M == 16)
+    {
+        auto const r = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+        return op(bits_as<T>((int) r[0]), bits_as<T>((int) r[1]));
+    }
+    else if constexpr (M == 32)
+    {
+        auto const r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+        return op(bits_as<T>((int) r[0]), bits_as<T>((int) r[1]));
+    }
+    else
+    {
+        // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror
+        constexpr int ctrl = M == 1 ? 0xB1 : (M == 2 ? 0x4E : (M == 4 ? 0x141 : 0x140));
+        static_assert(M == 1 || M == 2 || M == 4 || M == 8, "step");
+        return op(v, bits_as<T>(__builtin_amdgcn_update_dpp(bits, bits, ctrl, 0xF, 0xF, false)));
+    }
+}
+
+// The value held by the partner lane of step M (see reduce_step), for combinations that are not
+// symmetric in their operands.
+template <int M, typename T>
+__device__ inline T lane_partner(T v)
+{
+    static_assert(sizeof(T) == 4, "32-bit values");
+    int const bits = bits_as<int>(v);
+    if constexpr (M == 16 || M == 32)
+    {
+        // the swap leaves (own, other) in the two results for even rows / the low half and
+        // (other, own) for odd rows / the high half
+        int r0, r1;
+        if constexpr (M == 16)
+        {
+            auto const r = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+            r0 = (int) r[0];
+            r1 = (int) r[1];
+        }
+        else
+        {
+            auto const r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+            r0 = (int) r[0];
+            r1 = (int) r[1];
+        }
+        return bits_as<T>((threadIdx.x & M) ? r0 : r1);
+    }
+    else
+    {
+        constexpr int ctrl = M == 1 ? 0xB1 : (M == 2 ? 0x4E : (M == 4 ? 0x141 : 0x140));
+        static_assert(M == 1 || M == 2 || M == 4 || M == 8, "step");
+        return bits_as<T>(__builtin_amdgcn_update_dpp(bits, bits, ctrl, 0xF, 0xF, false));
+    }
+}
+
+// Butterfly over the SPAN lanes of a group (SPAN a power of two <= 64), starting at step FIRST.
+template <int SPAN, typename T, typename Op, int FIRST = 1>
+__device__ inline T group_allreduce(T v, Op op)
+{
+    if constexpr (FIRST < SPAN)
+    {
+        v = reduce_step<FIRST>(v, op);
+        return group_allreduce<SPAN, T, Op, FIRST * 2>(v, op);
+    }
+    else
+    {
+        return v;
+    }
+}
 
 __device__ inline float wave_sum(float v)
 {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1)
-    {
-        v += __shfl_xor(v, m, kWaveSize);
-    }
-    return v;
+    return group_allreduce<kWaveSize>(v, [](float a, float b) { return a + b; });
+}
+
+__device__ inline int wave_sum_i32(int v)
+{
+    return group_allreduce<kWaveSize>(v, [](int a, int b) { return a + b; });
 }
 
 __device__ inline float wave_max(float v)
 {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1)
-    {
-        v = fmaxf(v, __shfl_xor(v, m, kWaveSize));
-    }
-    return v;
+    return group_allreduce<kWaveSize>(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
 __device__ inline int wave_min_i32(int v)
 {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1)
-    {
-        v = min(v, __shfl_xor(v, m, kWaveSize));
-    }
-    return v;
+    return group_allreduce<kWaveSize>(v, [](int a, int b) { return min(a, b); });
 }
 
 // Running (count, mean, sum of squared deviations); merged pairwise with Chan's formula so the
@@ -78,21 +154,38 @@ __device__ inline Welford welford_merge(Welford a, Welford b)
 
 // Butterfly over `span` adjacent lanes (span a power of two <= 64); every lane of the group ends
 // with the group's statistics (taken from the group's first lane so all lanes agree bit for bit).
+template <int SPAN, int FIRST = 1>
+__device__ inline Welford welford_butterfly(Welford w)
+{
+    if constexpr (FIRST < SPAN)
+    {
+        Welford o;
+        o.n = lane_partner<FIRST>(w.n);
+        o.mean = lane_partner<FIRST>(w.mean);
+        o.m2 = lane_partner<FIRST>(w.m2);
+        return welford_butterfly<SPAN, FIRST * 2>(welford_merge(w, o));
+    }
+    else
+    {
+        return w;
+    }
+}
+
 template <int SPAN>
 __device__ inline Welford group_welford(Welford w)
 {
-#pragma unroll
-    for (int m = SPAN / 2; m >= 1; m >>= 1)
+    w = welford_butterfly<SPAN>(w);
+    if constexpr (SPAN == kWaveSize)
     {
-        Welford o;
-        o.n = __shfl_xor(w.n, m, kWaveSize);
-        o.mean = __shfl_xor(w.mean, m, kWaveSize);
-        o.m2 = __shfl_xor(w.m2, m, kWaveSize);
-        w = welford_merge(w, o);
+        w.mean = bits_as<float>(__builtin_amdgcn_readfirstlane(bits_as<int>(w.mean)));
+        w.m2 = bits_as<float>(__builtin_amdgcn_readfirstlane(bits_as<int>(w.m2)));
     }
-    int const lead = (threadIdx.x & (kWaveSize - 1)) & ~(SPAN - 1);
-    w.mean = __shfl(w.mean, lead, kWaveSize);
-    w.m2 = __shfl(w.m2, lead, kWaveSize);
+    else
+    {
+        int const lead = (threadIdx.x & (kWaveSize - 1)) & ~(SPAN - 1);
+        w.mean = __shfl(w.mean, lead, kWaveSize);
+        w.m2 = __shfl(w.m2, lead, kWaveSize);
+    }
     return w;
 }
 

@@ -441,8 +441,8 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
                 }
             }
         }
-        mx = max(mx, __shfl_xor(mx, 16, kWaveSize));
-        mx = max(mx, __shfl_xor(mx, 32, kWaveSize));
+        mx = reduce_step<16>(mx, [](int x, int y) { return max(x, y); });
+        mx = reduce_step<32>(mx, [](int x, int y) { return max(x, y); });
 
         // ---- e = 2^((acc - max) * c), row sum; a fully masked row has max = -inf -> all e = 0 --
         float const negK0 = mx == kNegInfBits ? 0.f : -__int_as_float(mx) * a.c;
@@ -471,8 +471,8 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
                 }
             }
         }
-        sum += __shfl_xor(sum, 16, kWaveSize);
-        sum += __shfl_xor(sum, 32, kWaveSize);
+        sum = reduce_step<16>(sum, [](float x, float y) { return x + y; });
+        sum = reduce_step<32>(sum, [](float x, float y) { return x + y; });
         float const r = sum > 0.f ? a.scaleSoftmax / sum : 0.f;
         // e * r <= scale_softmax: only a scale above 127 can leave the INT8 range; the row is then
         // pre-clamped through e <= 127 / r (one extra op per score on that rare path only)
@@ -816,8 +816,8 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
             mxB = max(max(mxB, acc[t][2]), acc[t][3]);
         }
         int mx = max(mxA, mxB);
-        mx = max(mx, __shfl_xor(mx, 16, kWaveSize));
-        mx = max(mx, __shfl_xor(mx, 32, kWaveSize));
+        mx = reduce_step<16>(mx, [](int x, int y) { return max(x, y); });
+        mx = reduce_step<32>(mx, [](int x, int y) { return max(x, y); });
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- e = 2^((acc - max) * c) in place, row sum
@@ -850,8 +850,8 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
             }
         }
         float sum = sum0 + sum1;
-        sum += __shfl_xor(sum, 16, kWaveSize);
-        sum += __shfl_xor(sum, 32, kWaveSize);
+        sum = reduce_step<16>(sum, [](float x, float y) { return x + y; });
+        sum = reduce_step<32>(sum, [](float x, float y) { return x + y; });
         float const r = a.scaleSoftmax / sum;   // sum >= 1: the row maximum contributes 2^0
 
         // ---- p8 = rne(e * r), four keys to a dword; O^T = V^T P^T
@@ -1143,8 +1143,8 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
                 }
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, kWaveSize));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWaveSize));
+        mx = reduce_step<16>(mx, [](float x, float y) { return fmaxf(x, y); });
+        mx = reduce_step<32>(mx, [](float x, float y) { return fmaxf(x, y); });
 
         // ---- p = 2^((s - max) * c) rounded to binary16; O^T = V^T P^T; the row sum is taken by
         //      the matrix unit as well (a tile of ones), so numerator and denominator see the
@@ -1369,8 +1369,8 @@ __device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq,
             mxB = fmaxf(fmaxf(mxB, acc[t][2]), acc[t][3]);
         }
         float mx = fmaxf(mxA, mxB);
-        mx = fmaxf(mx, __shfl_xor(mx, 16, kWaveSize));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWaveSize));
+        mx = reduce_step<16>(mx, [](float x, float y) { return fmaxf(x, y); });
+        mx = reduce_step<32>(mx, [](float x, float y) { return fmaxf(x, y); });
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- p = 2^((s - max) * c) rounded to binary16; O^T = V^T P^T; row sum by a tile of ones

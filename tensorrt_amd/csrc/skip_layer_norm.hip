@@ -356,15 +356,11 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
                 }
             }
         }
-#pragma unroll
-        for (int m = 1; m < kWaveSize; m *= 2)
-        {
-            sIn += __shfl_xor(sIn, m, kWaveSize);
-            sSk += __shfl_xor(sSk, m, kWaveSize);
-            sII += __shfl_xor(sII, m, kWaveSize);
-            sIS += __shfl_xor(sIS, m, kWaveSize);
-            sSS += __shfl_xor(sSS, m, kWaveSize);
-        }
+        sIn = wave_sum_i32(sIn);
+        sSk = wave_sum_i32(sSk);
+        sII = wave_sum_i32(sII);
+        sIS = wave_sum_i32(sIS);
+        sSS = wave_sum_i32(sSS);
         double sum1 = dIn * sIn + dSk * sSk;
         double sum2 = dIn * dIn * sII + 2.0 * dIn * dSk * sIS + dSk * dSk * sSS;
         if (HAS_BIAS)
@@ -479,14 +475,25 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
         }
     }
     // the lanes of a token differ in bit 0 (half) and in the sub bits above the token bits
-#pragma unroll
-    for (int m = 1; m < kWaveSize; m = (m == 1 ? LPG : m * 2))
     {
-        sIn += __shfl_xor(sIn, m, kWaveSize);
-        sSk += __shfl_xor(sSk, m, kWaveSize);
-        sII += __shfl_xor(sII, m, kWaveSize);
-        sIS += __shfl_xor(sIS, m, kWaveSize);
-        sSS += __shfl_xor(sSS, m, kWaveSize);
+        auto const add = [](int x, int y) { return x + y; };
+        auto const over_token = [&](int v) {
+            v = reduce_step<1>(v, add);
+            if constexpr (LPG <= 16)
+            {
+                v = reduce_step<16>(v, add);
+            }
+            if constexpr (LPG <= 32)
+            {
+                v = reduce_step<32>(v, add);
+            }
+            return v;
+        };
+        sIn = over_token(sIn);
+        sSk = over_token(sSk);
+        sII = over_token(sII);
+        sIS = over_token(sIS);
+        sSS = over_token(sSS);
     }
     if (W > 1)
     {
