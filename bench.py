@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 METRIC = "BERT-large INT8 S=384 seq/s on 1 GPU; % HBM peak (LN) & % INT8 MFMA peak (MHA)"
 PEAK_INT8_OPS = 5.0e15   # dense INT8 MFMA, op/s
 PEAK_HBM = 8.0e12        # B/s
+# HBM bytes per launch on the default workload, from the FETCH_SIZE / WRITE_SIZE counter runs kept in
+# profiles/ (scaled by what the same counters read for a 256 MiB copy); null for any other workload.
+MHA_TRAFFIC_BYTES = 75_200_000
+LN_TRAFFIC_BYTES = 59_700_000
 
 
 def f32_bits(x) -> int:
@@ -175,6 +179,26 @@ def main():
     t_mha = kernel_time(mha)
     t_ln = kernel_time(skipln)
 
+    # The LayerNorm tensors (56 MB) fit in the 256 MB last-level cache, so back-to-back launches on
+    # the same buffers are partly served from it.  Cold figure: rotate over enough buffer sets that a
+    # set has been evicted before it is touched again (6 x 56 MB).
+    sets = []
+    for _ in range(6):
+        sets.append((torch.randint(-127, 128, (T * E,), dtype=torch.int8, device="cuda"),
+                     torch.randint(-127, 128, (T * E,), dtype=torch.int8, device="cuda"),
+                     torch.empty(T * E, dtype=torch.int8, device="cuda")))
+    turn = [0]
+
+    def skipln_cold():
+        a_in, a_skip, a_out = sets[turn[0] % len(sets)]
+        turn[0] += 1
+        api.check(api.skipln_interleaved_large_hface(stream, E, T, a_in.data_ptr(), a_skip.data_ptr(),
+                                                      d["beta"].data_ptr(), d["gamma"].data_ptr(), a_out.data_ptr(),
+                                                      s_ctx, wl.s_skip, q_out))
+
+    t_ln_cold = kernel_time(skipln_cold)
+    del sets
+
     if args.pmc_calibration:
         src = torch.zeros(256 << 20, dtype=torch.int8, device="cuda")
         dst = torch.empty_like(src)
@@ -184,6 +208,7 @@ def main():
 
     mha_ops = wl.mha_ops()
     ln_bytes = wl.skipln_bytes(1)
+    default_workload = (args.batch, args.seqlen, args.seed) == (64, 384, 1)
     out = {
         "metric": METRIC,
         "value": round(wl.B / (ms_step * 1e-3), 1),
@@ -211,7 +236,7 @@ def main():
             "peak": PEAK_INT8_OPS / 1e12,
             "unit": "TOP/s",
             "frac": round(mha_ops / t_mha / PEAK_INT8_OPS, 4),
-            "traffic": None,
+            "traffic": MHA_TRAFFIC_BYTES if default_workload else None,
             "avg_launch_us": round(t_mha * 1e6, 2),
             "algorithmic_ops_per_launch": mha_ops,
             "hbm_frac": round(wl.mha_bytes() / t_mha / PEAK_HBM, 4),
@@ -223,9 +248,13 @@ def main():
             "peak": PEAK_HBM / 1e9,
             "unit": "GB/s",
             "frac": round(ln_bytes / t_ln / PEAK_HBM, 4),
-            "traffic": None,
+            "traffic": LN_TRAFFIC_BYTES if default_workload else None,
             "avg_launch_us": round(t_ln * 1e6, 2),
             "algorithmic_bytes_per_launch": ln_bytes,
+            "cold_cache": {"achieved": round(ln_bytes / t_ln_cold / 1e9, 1), "frac": round(ln_bytes / t_ln_cold / PEAK_HBM, 4),
+                           "avg_launch_us": round(t_ln_cold * 1e6, 2),
+                           "how": "6 rotating buffer sets (336 MB) so that no launch finds its tensors in the "
+                                  "256 MB last-level cache"},
         },
     }
     if not args.no_cpu_baseline:
