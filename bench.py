@@ -230,7 +230,7 @@ def main():
             "lengths": f"uniform[{wl.S // 2},{wl.S}] seed {args.seed}",
         },
         "roofline": {
-            "kernel": "fmha_i8_kernel (interleaved)",
+            "kernel": "fmha_i8_prefix_kernel<6,true>",
             "bound": "mfma",
             "achieved": round(mha_ops / t_mha / 1e12, 2),
             "peak": PEAK_INT8_OPS / 1e12,
@@ -242,7 +242,7 @@ def main():
             "hbm_frac": round(wl.mha_bytes() / t_mha / PEAK_HBM, 4),
         },
         "roofline_skipln": {
-            "kernel": "skipln_interleaved_kernel<32,false>",
+            "kernel": "skipln_interleaved_kernel<32,8,32,false>",
             "bound": "hbm",
             "achieved": round(ln_bytes / t_ln / 1e9, 1),
             "peak": PEAK_HBM / 1e9,
