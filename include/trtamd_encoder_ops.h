@@ -1,0 +1,62 @@
+/*
+ * C-ABI of the encoder operations that sit BETWEEN the BERT plugins in a TensorRT engine: the INT8
+ * linear layers (QKV projection, attention output projection, the two feed-forward layers) and the
+ * layout / quantisation reformats either side of the interleaved plugins.  In the reference these
+ * are not plugin code: TensorRT's closed core executes them (the only open counterpart is the
+ * deprecated cuBLASLt plugin plugin/fcPlugin, FP32/FP16 only, plugin/fcPlugin/README.md:41-45), so
+ * the semantics below are this library's own statement of an INT8 fully-connected layer with
+ * folded quantisation scales.  Same calling rules as trtamd_bert_kernels.h: plain device pointers,
+ * asynchronous on the given stream, int status, nothing allocates or synchronises.
+ */
+#ifndef TRTAMD_ENCODER_OPS_H
+#define TRTAMD_ENCODER_OPS_H
+
+#include "trtamd_bert_kernels.h"
+
+#ifdef __cplusplus
+extern "C"
+{
+#endif
+
+/* What happens to the INT32 accumulator acc[t][n] = sum_k a[t][k] * w[n][k] (exact). */
+enum
+{
+    /* y = fmaf(float(acc), alpha[n], beta[n]);  out8 = sat8(rne(y)).  alpha = s_a * s_w[n] / s_out and
+     * beta = bias[n] / s_out: the caller folds the output scale, as a TensorRT build does. */
+    TRTAMD_LINEAR_AFFINE = 0,
+    /* y as above with alpha = s_a * s_w[n], beta = bias[n];  g = 0.5 * y * (1 + erf(y / sqrt(2)));
+     * out8 = sat8(rne(g * out_scale)), out_scale = 1 / s_out. */
+    TRTAMD_LINEAR_GELU = 1,
+    /* out32[t][n] = acc, linear layout: the accumulators themselves, for bit-exact checks. */
+    TRTAMD_LINEAR_RAW_INT32 = 2,
+    /* out16[t][n] = binary16(y), linear layout: the de-quantised result (e.g. the last layer). */
+    TRTAMD_LINEAR_AFFINE_FP16 = 3
+};
+
+typedef struct trtamd_int8_linear_params
+{
+    int8_t const* a;    /* activations: linear [T][K], or 32-interleaved [K/32][T][32] */
+    int8_t const* w;    /* weights: linear [N][K] (one row of K per output channel), or 32-interleaved
+                           [K/32][N][32] (the faster one: a build step reformats constant weights once).  For the QKV
+                           projection the rows are ordered [head][q|k|v][64], the packing
+                           plugin/bertQKVToContextPlugin/README.md:27-30 asks for. */
+    float const* alpha; /* [N] */
+    float const* beta;  /* [N] */
+    void* out;          /* int8 [T][N] or [N/32][T][32]; int32 / binary16 [T][N] */
+    int32_t T, K, N;    /* K % 64 == 0, N % 32 == 0 */
+    int32_t a_interleaved;
+    int32_t w_interleaved;
+    int32_t out_interleaved;
+    int32_t epilogue;
+    float out_scale;    /* TRTAMD_LINEAR_GELU only */
+} trtamd_int8_linear_params;
+
+/* Stands where TensorRT's own INT8 fully-connected / 1x1-convolution layer runs between the plugins
+ * (closed source; engine-side placement described in plugin/bertQKVToContextPlugin/README.md:25-30). */
+TRTAMD_API int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_params const* params);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TRTAMD_ENCODER_OPS_H */

@@ -300,3 +300,37 @@ def zero_padding_2d(src_bytes, spitch, dpitch, height):
     dst = np.empty(height * dpitch, np.uint8)
     lib().orc_zero_padding_2d(_p(src), _p(dst), C.c_int64(height), C.c_int(spitch), C.c_int(dpitch), C.c_int(1))
     return dst
+
+
+# ------------------------------------------------------------------------------------------------
+# INT8 linear layer between the plugins
+# ------------------------------------------------------------------------------------------------
+
+LINEAR_AFFINE, LINEAR_GELU, LINEAR_RAW_INT32, LINEAR_AFFINE_FP16 = 0, 1, 2, 3
+
+
+def int8_linear(a, w, alpha=None, beta=None, epilogue=LINEAR_AFFINE, out_scale=1.0, a_interleaved=False,
+                out_interleaved=False):
+    """a: int8 [T,K] (or [K/32,T,32] if a_interleaved); w: int8 [N,K]; alpha, beta: float32 [N].
+
+    Returns int8 [T,N] (or [N/32,T,32] if out_interleaved), int32 [T,N] for LINEAR_RAW_INT32,
+    float16 [T,N] for LINEAR_AFFINE_FP16.
+    """
+    a = _c(a, np.int8)
+    w = _c(w, np.int8)
+    N, K = w.shape
+    T = a.shape[1] if a_interleaved else a.shape[0]
+    alpha = _c(alpha, np.float32)
+    beta = _c(beta, np.float32)
+    if epilogue == LINEAR_RAW_INT32:
+        out = np.zeros((T, N), np.int32)
+    elif epilogue == LINEAR_AFFINE_FP16:
+        out = np.zeros((T, N), np.float16)
+    else:
+        out = np.zeros((N // 32, T, 32) if out_interleaved else (T, N), np.int8)
+    rc = lib().orc_int8_linear(C.c_int64(T), C.c_int(K), C.c_int(N), _p(a), C.c_int(int(a_interleaved)), _p(w),
+                               _p(alpha), _p(beta), C.c_int(epilogue), C.c_float(out_scale),
+                               C.c_int(int(out_interleaved)), _p(out))
+    if rc != 0:
+        raise ValueError("orc_int8_linear rejected its arguments")
+    return out

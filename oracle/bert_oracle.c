@@ -1101,3 +1101,63 @@ ORC_API void orc_zero_padding_2d(void const* src, void* dst, int64_t rows, int s
         }
     }
 }
+
+/* INT8 linear layer between the plugins (QKV / output projection / feed-forward).  There is no open
+ * reference source for it (TensorRT's closed core runs these layers; plugin/fcPlugin is the FP16/FP32
+ * cuBLASLt stand-in, plugin/fcPlugin/README.md:41-45), so this states the arithmetic the library
+ * documents in include/trtamd_encoder_ops.h:
+ *   acc[t][n] = sum_k a[t][k] * w[n][k]                    exact INT32
+ *   y         = fmaf((float) acc, alpha[n], beta[n])        one binary32 rounding
+ *   epilogue 0: out8 = sat8(rne(y))
+ *   epilogue 1: g = 0.5 * y * (1 + erf(y / sqrt 2)) evaluated in binary64 and rounded to binary32,
+ *               out8 = sat8(rne(g * out_scale))
+ *   epilogue 2: out32 = acc           epilogue 3: out16 = binary16(y)
+ * Activations / INT8 outputs are linear [T][C] or 32-interleaved [C/32][T][32]
+ * (layout of qkvToContextInt8InterleavedPlugin.cpp:124-127); weights are [N][K] with the QKV rows in
+ * the [head][3][64] order of plugin/bertQKVToContextPlugin/README.md:27-30. */
+ORC_API int orc_int8_linear(int64_t T, int K, int N, int8_t const* a, int aInterleaved, int8_t const* w,
+    float const* alpha, float const* beta, int epilogue, float outScale, int outInterleaved, void* out)
+{
+    if (K <= 0 || N <= 0 || epilogue < 0 || epilogue > 3)
+    {
+        return 1;
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t)
+    {
+        int8_t* row = (int8_t*) malloc((size_t) K);
+        for (int k = 0; k < K; ++k)
+        {
+            row[k] = aInterleaved ? a[il_index(k, t, T)] : a[t * K + k];
+        }
+        for (int n = 0; n < N; ++n)
+        {
+            int8_t const* wr = w + (int64_t) n * K;
+            int32_t acc = 0;
+            for (int k = 0; k < K; ++k)
+            {
+                acc += (int32_t) row[k] * (int32_t) wr[k];
+            }
+            if (epilogue == 2)
+            {
+                ((int32_t*) out)[t * N + n] = acc;
+                continue;
+            }
+            float const y = fmaf((float) acc, alpha[n], beta[n]);
+            if (epilogue == 3)
+            {
+                ((uint16_t*) out)[t * N + n] = d2h((double) y);
+                continue;
+            }
+            float r = y;
+            if (epilogue == 1)
+            {
+                float const g = (float) (0.5 * (double) y * (1.0 + erf((double) y * 0.70710678118654752440)));
+                r = g * outScale;
+            }
+            ((int8_t*) out)[outInterleaved ? il_index(n, t, T) : t * N + n] = sat8_rne(r);
+        }
+        free(row);
+    }
+    return 0;
+}

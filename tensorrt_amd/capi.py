@@ -31,6 +31,18 @@ class FmhaParams(C.Structure):
     ]
 
 
+class Int8LinearParams(C.Structure):
+    """struct trtamd_int8_linear_params (include/trtamd_encoder_ops.h)."""
+    _fields_ = [
+        ("a", c_p), ("w", c_p), ("alpha", c_p), ("beta", c_p), ("out", c_p),
+        ("T", i32), ("K", i32), ("N", i32),
+        ("a_interleaved", i32), ("w_interleaved", i32), ("out_interleaved", i32), ("epilogue", i32),
+        ("out_scale", f32),
+    ]
+
+
+LINEAR_AFFINE, LINEAR_GELU, LINEAR_RAW_INT32, LINEAR_AFFINE_FP16 = 0, 1, 2, 3
+
 _SIGS = {
     "trtamd_version": (C.c_int, []),
     "trtamd_last_error": (C.c_char_p, []),
@@ -63,10 +75,13 @@ _SIGS = {
     "trtamd_fused_mha_run_debug": (C.c_int, [c_p, i32, C.POINTER(FmhaParams), c_p, c_p]),
     "trtamd_fused_mha_is_valid": (C.c_int, [i32, i32, i32]),
     "trtamd_zero_padding_2d": (C.c_int, [c_p, i32, c_p, i32, i32, c_p]),
+    "trtamd_int8_linear": (C.c_int, [c_p, C.POINTER(Int8LinearParams)]),
 }
 
 # Entry points declared in include/trtamd_bert_kernels.h (the debug hook is extra).
-HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug"]
+# Entry points declared in include/trtamd_encoder_ops.h.
+ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear"]
+HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug" and k not in ENCODER_OPS_SYMBOLS]
 
 
 class TrtAmdError(RuntimeError):

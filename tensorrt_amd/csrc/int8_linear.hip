@@ -1,0 +1,468 @@
+// INT8 linear layer for gfx950: out[t][n] = epilogue(sum_k a[t][k] * w[n][k]).
+//
+// The projections between the encoder plugins (QKV, attention output, the two feed-forward
+// layers) are plain GEMMs whose operands are both contiguous along k, which is what the INT8 MFMA
+// wants: a lane feeds 16 consecutive k-bytes of one row.  v_mfma_i32_32x32x32_i8 is used because it
+// runs at the full INT8 rate of the matrix core (measured: 32768 MACs in 33 cycles per SIMD);
+// v_mfma_i32_16x16x64_i8 takes 32 cycles for half as many.  The kernel computes the transposed
+// product (output channels are the M dimension, tokens the N dimension) so that a lane ends up with
+// groups of four consecutive channels of one token, which pack into the token-major INT8 output of
+// either layout.
+//
+// Tiling: a workgroup owns BM channels x BN tokens, its waves a WM x WN grid of (MT*32) x (NT*32)
+// sub-tiles kept in INT32 accumulators.  One stage is 64 bytes of k for the whole tile (two MFMA
+// steps).  Global loads are 16 bytes per lane with consecutive lanes on consecutive addresses; a
+// fragment sits in LDS row-major with a one-bit swizzle, so LDS writes and the 16-byte-per-lane
+// fragment reads are both conflict-free.  Stages are double-buffered in LDS and the loads run two
+// stages ahead of the multiplication through two register sets.
+//
+// Activations, weights and outputs may be in the linear layout [R][C] or in the 32-interleaved
+// layout [C/32][R][32] that the interleaved encoder plugins use; the interleaved one makes every
+// load unit 1 KB of contiguous memory.
+#include "device_utils.hpp"
+#include "host_utils.hpp"
+#include "trtamd_encoder_ops.h"
+
+#include <cstdlib>
+#include <type_traits>
+
+namespace trtamd
+{
+namespace
+{
+
+constexpr float kRoundMagic = 12582912.f; // 1.5 * 2^23: adding it rounds to nearest even
+constexpr int kRoundMagicBits = 0x4B400000;
+
+enum Epilogue
+{
+    kAFFINE = TRTAMD_LINEAR_AFFINE,
+    kGELU = TRTAMD_LINEAR_GELU,
+    kRAW = TRTAMD_LINEAR_RAW_INT32,
+    kHALF = TRTAMD_LINEAR_AFFINE_FP16
+};
+
+struct LinearArgs
+{
+    int8_t const* a;
+    int8_t const* w;
+    float const* alpha;
+    float const* beta;
+    void* out;
+    int T, K, N;
+    float qOut;
+};
+
+// 0.5 * erfc(|y| / sqrt(2)) by the rational-exponential form of Abramowitz & Stegun 7.1.26
+// (absolute error below 1e-7), then gelu(y) = max(y, 0) - |y| * that.
+__device__ inline float gelu_erf(float y)
+{
+    float const ay = fabsf(y);
+    float const x = ay * 0.70710678f;
+    float const t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, x, 1.0f));
+    float p = fmaf(t, 0.5f * 1.061405429f, 0.5f * -1.453152027f);
+    p = fmaf(p, t, 0.5f * 1.421413741f);
+    p = fmaf(p, t, 0.5f * -0.284496736f);
+    p = fmaf(p, t, 0.5f * 0.254829592f);
+    p *= t;
+    float const u = ay * 0.84932180f; // |y| / sqrt(2) * sqrt(log2 e)
+    float const e = __builtin_amdgcn_exp2f(-(u * u));
+    return fmaf(-ay, p * e, fmaxf(y, 0.f));
+}
+
+// Bits of (v + 1.5*2^23) clamped so that the low byte is sat8(rne(v)).
+__device__ inline uint32_t round_sat8_bits(float v)
+{
+    int const b = bits_as<int>(v + kRoundMagic);
+    return (uint32_t) min(max(b, kRoundMagicBits - 128), kRoundMagicBits + 127);
+}
+
+__device__ inline uint32_t low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3)
+{
+    uint32_t const lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
+    uint32_t const hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
+// One operand fragment of v_mfma_i32_32x32x32_i8 is 32 rows x 32 k-bytes; lane l feeds row l%32,
+// bytes 16*(l/32)..+15.  In LDS a fragment is 1 KB, row-major, with the two 16-byte halves of a row
+// swapped for rows 8..15 and 24..31: a 16-lane group then reads 16 different 16-byte columns of the
+// bank array, and so does a group that writes 8 whole rows.
+__device__ inline int frag_offset(int row, int half)
+{
+    return row * 32 + ((half ^ ((row >> 3) & 1)) << 4);
+}
+
+template <int WM, int WN, int MT, int NT, bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
+__global__ __launch_bounds__(64 * WM * WN) void int8_linear_kernel(LinearArgs const p)
+{
+    constexpr int NWAVES = WM * WN;
+    constexpr int BM = WM * MT * 32;    // output channels per workgroup
+    constexpr int BN = WN * NT * 32;    // tokens per workgroup
+    constexpr int AF = (BM / 32) * 2;   // weight fragments per stage (64 bytes of k = two MFMA steps)
+    constexpr int BF = (BN / 32) * 2;   // activation fragments per stage
+    static_assert(AF % NWAVES == 0 && BF % NWAVES == 0, "load units divide evenly among the waves");
+    constexpr int LA = AF / NWAVES;
+    constexpr int LB = BF / NWAVES;
+    constexpr int STAGE = (AF + BF) * 1024;
+
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
+    __shared__ __attribute__((aligned(16))) float sAlpha[BM];
+    __shared__ __attribute__((aligned(16))) float sBeta[BM];
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const wm = wave / WN;
+    int const wn = wave % WN;
+    int const col32 = lane & 31;
+    int const hi = lane >> 5;
+
+    // channel tiles vary fastest, so the workgroups resident on one XCD share a few token tiles
+    // (read from HBM once into that XCD's L2) and sweep all the weights
+    uint32_t const nbm = (uint32_t) ((p.N + BM - 1) / BM);
+    uint32_t const tile = xcd_remap(blockIdx.x, gridDim.x);
+    int const n0 = (int) (tile % nbm) * BM;
+    int const t0 = (int) (tile / nbm) * BN;
+
+    // A load unit is 1 KB that one wave fetches with one 16-byte load per lane, consecutive lanes
+    // reading consecutive memory.  Interleaved operand [K/32][R][32]: unit (rb, ks) is the 32 rows of
+    // row block rb in k-slab ks, contiguous in memory, and is exactly one fragment.  Linear operand
+    // [R][K]: unit (rb, h) is rows 16h..16h+15 of the block, 64 bytes of k each, and lands in the two
+    // fragments (rb, 0) and (rb, 1).
+    auto unit_addressing = [&](bool interleaved, int unit, int row0, int R, uint32_t& gOff, int& lOff) {
+        int const rb = unit >> 1, sel = unit & 1;
+        if (interleaved)
+        {
+            int const r = lane >> 1, c = lane & 1;
+            int const row = min(row0 + rb * 32 + r, R - 1);
+            gOff = ((uint32_t) sel * (uint32_t) R + (uint32_t) row) * 32u + (uint32_t) c * 16u;
+            lOff = (rb * 2 + sel) * 1024 + frag_offset(r, c);
+        }
+        else
+        {
+            int const r = sel * 16 + (lane >> 2), c = lane & 3;
+            int const row = min(row0 + rb * 32 + r, R - 1);
+            gOff = (uint32_t) row * (uint32_t) p.K + (uint32_t) c * 16u;
+            lOff = (rb * 2 + (c >> 1)) * 1024 + frag_offset(r, c & 1);
+        }
+    };
+    uint32_t offA[LA], offB[LB];
+    int ldsA[LA], ldsB[LB];
+#pragma unroll
+    for (int q = 0; q < LA; ++q)
+    {
+        unit_addressing(IL_W, q * NWAVES + wave, n0, p.N, offA[q], ldsA[q]);
+    }
+#pragma unroll
+    for (int q = 0; q < LB; ++q)
+    {
+        unit_addressing(IL_IN, q * NWAVES + wave, t0, p.T, offB[q], ldsB[q]);
+        ldsB[q] += AF * 1024;
+    }
+    uint32_t const stepA = IL_W ? 2u * (uint32_t) p.N * 32u : 64u;
+    uint32_t const stepB = IL_IN ? 2u * (uint32_t) p.T * 32u : 64u;
+
+    // two register sets: the loads of stage s+2 are issued while stage s is multiplied, so a load has
+    // two stages of MFMA work to hide behind before its data is moved to LDS
+    i32x4 ga[2][LA], gb[2][LB];
+    auto fetch = [&](auto set, int kt) {
+        constexpr int S = decltype(set)::value;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            ga[S][q] = *reinterpret_cast<i32x4 const*>(p.w + offA[q] + (uint32_t) kt * stepA);
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            gb[S][q] = *reinterpret_cast<i32x4 const*>(p.a + offB[q] + (uint32_t) kt * stepB);
+        }
+    };
+    auto stash = [&](auto set, int buf) {
+        constexpr int S = decltype(set)::value;
+        uint8_t* base = lds + buf * STAGE;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            *reinterpret_cast<i32x4*>(base + ldsA[q]) = ga[S][q];
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            *reinterpret_cast<i32x4*>(base + ldsB[q]) = gb[S][q];
+        }
+    };
+
+    i32x16 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+    {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+        {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+            {
+                acc[i][j][v] = 0;
+            }
+        }
+    }
+    int const readOff = frag_offset(col32, hi);
+    auto multiply = [&](int buf) {
+        uint8_t const* base = lds + buf * STAGE + readOff;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+        {
+            i32x4 fa[MT], fb[NT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+            {
+                fa[i] = *reinterpret_cast<i32x4 const*>(base + ((wm * MT + i) * 2 + ks) * 1024);
+            }
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+            {
+                fb[j] = *reinterpret_cast<i32x4 const*>(base + (AF + (wn * NT + j) * 2 + ks) * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+            {
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+    };
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, 1>;
+
+    // per-channel scale and offset of the tile, staged once for the epilogue
+    if constexpr (EPI != kRAW)
+    {
+        for (int c = threadIdx.x; c < BM; c += 64 * NWAVES)
+        {
+            int const n = min(n0 + c, p.N - 1);
+            sAlpha[c] = p.alpha[n];
+            sBeta[c] = p.beta[n];
+        }
+    }
+
+    // Stage kt sits in LDS buffer kt&1 and arrived through register set kt&1.  The loop body has no
+    // branches (loads past the last stage re-read the last stage and are never used), so the number of
+    // loads in flight at every point is fixed and a stash waits for its own four loads only.
+    int const nk = p.K / 64;
+    fetch(Set0{}, 0);
+    fetch(Set1{}, min(1, nk - 1));
+    stash(Set0{}, 0);
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2)
+    {
+        fetch(Set0{}, min(kt + 2, nk - 1));
+        multiply(0);
+        stash(Set1{}, 1);
+        __syncthreads();
+        fetch(Set1{}, min(kt + 3, nk - 1));
+        multiply(1);
+        stash(Set0{}, 0);
+        __syncthreads();
+    }
+    if (kt < nk)
+    {
+        multiply(0);
+    }
+
+    // ---- epilogue -------------------------------------------------------------------------------
+    // Accumulator register v of a 32x32 tile is token l%32, channel 8*(v/4) + 4*(l/32) + v%4: four
+    // groups of four consecutive channels.  For the INT8 outputs the two lanes that share a token
+    // trade two packed dwords (v_permlane32_swap), after which lane l holds the 16 consecutive
+    // channels 16*(l/32)..+15 and stores them with one 16-byte write.
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+    {
+        int const cl = (wm * MT + i) * 32; // wave-uniform, and so is the guard: N is a multiple of 32
+        if (n0 + cl >= p.N)
+        {
+            break;
+        }
+        f32x4 al[4], be[4];
+        if constexpr (EPI != kRAW)
+        {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + cl + 8 * g + 4 * hi);
+                be[g] = *reinterpret_cast<f32x4 const*>(sBeta + cl + 8 * g + 4 * hi);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+        {
+            int const t = t0 + (wn * NT + j) * 32 + col32;
+            bool const live = t < p.T;
+            if constexpr (EPI == kRAW)
+            {
+                if (live)
+                {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        i32x4 const v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                            acc[i][j][4 * g + 3]};
+                        *reinterpret_cast<i32x4*>(
+                            static_cast<int32_t*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
+                            = v;
+                    }
+                }
+            }
+            else if constexpr (EPI == kHALF)
+            {
+                if (live)
+                {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        f16x4 h;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            h[e] = (f16) fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
+                        }
+                        *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
+                            = h;
+                    }
+                }
+            }
+            else
+            {
+                int d[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    uint32_t b[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        float y = fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
+                        if constexpr (EPI == kGELU)
+                        {
+                            y = gelu_erf(y) * p.qOut;
+                        }
+                        b[e] = round_sat8_bits(y);
+                    }
+                    d[g] = (int) low_bytes(b[0], b[1], b[2], b[3]);
+                }
+                // lanes l < 32 hold channels [0-3][8-11][16-19][24-27], lanes l+32 the gaps
+                auto const s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                auto const s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+                i32x4 const packed = {(int) s02[0], (int) s02[1], (int) s13[0], (int) s13[1]};
+                if (live)
+                {
+                    int const c = n0 + cl + 16 * hi;
+                    size_t const o = IL_OUT ? ((size_t) (c >> 5) * p.T + t) * 32 + (c & 31) : (size_t) t * p.N + c;
+                    *reinterpret_cast<i32x4*>(static_cast<int8_t*>(p.out) + o) = packed;
+                }
+            }
+        }
+    }
+}
+
+template <int WM, int WN, int MT, int NT, bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
+int launch_tile(hipStream_t stream, LinearArgs const& a)
+{
+    constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
+    uint32_t const grid = (uint32_t) ceil_div(a.N, BM) * (uint32_t) ceil_div(a.T, BN);
+    hipLaunchKernelGGL((int8_linear_kernel<WM, WN, MT, NT, IL_W, IL_IN, IL_OUT, EPI>), dim3(grid), dim3(64 * WM * WN),
+        0, stream, a);
+    return check_launch("int8_linear_kernel");
+}
+
+template <bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
+int launch_shape(hipStream_t stream, LinearArgs const& a)
+{
+    static int const forced = [] {
+        char const* e = getenv("TRTAMD_LINEAR_TILE");
+        return e ? atoi(e) : -1;
+    }();
+    // large problems: 256 channels x 256 tokens per workgroup; small ones: 128 x 128 so that the
+    // launch still has a workgroup for every CU
+    int64_t const big = (int64_t) ceil_div(a.N, 256) * ceil_div(a.T, 256);
+    int const choice = forced >= 0 ? forced : (big >= 256 ? 0 : 1);
+    switch (choice)
+    {
+    case 0: return launch_tile<2, 4, 4, 2, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
+    case 1: return launch_tile<2, 2, 2, 2, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
+    case 2: return launch_tile<4, 2, 2, 4, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
+    case 3: return launch_tile<2, 2, 4, 2, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
+    case 4: return launch_tile<2, 2, 2, 4, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
+    default: return set_error(TRTAMD_STATUS_BAD_PARAM, "TRTAMD_LINEAR_TILE=%d is not a tile configuration", choice);
+    }
+}
+
+template <bool IL_W, bool IL_IN>
+int launch_out(hipStream_t stream, LinearArgs const& a, int epilogue, bool ilOut)
+{
+    switch (epilogue)
+    {
+    case kAFFINE:
+        return ilOut ? launch_shape<IL_W, IL_IN, true, kAFFINE>(stream, a)
+                     : launch_shape<IL_W, IL_IN, false, kAFFINE>(stream, a);
+    case kGELU:
+        return ilOut ? launch_shape<IL_W, IL_IN, true, kGELU>(stream, a)
+                     : launch_shape<IL_W, IL_IN, false, kGELU>(stream, a);
+    case kRAW: return launch_shape<IL_W, IL_IN, false, kRAW>(stream, a);
+    case kHALF: return launch_shape<IL_W, IL_IN, false, kHALF>(stream, a);
+    default: return set_error(TRTAMD_STATUS_BAD_PARAM, "int8_linear: unknown epilogue %d", epilogue);
+    }
+}
+
+} // namespace
+} // namespace trtamd
+
+extern "C" int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_params const* p)
+{
+    using namespace trtamd;
+    if (p == nullptr || p->a == nullptr || p->w == nullptr || p->out == nullptr)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "int8_linear: null pointer");
+    }
+    if (p->T < 0 || p->K <= 0 || p->N <= 0 || p->K % 64 != 0 || p->N % 32 != 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "int8_linear: T=%d K=%d N=%d (K must be a multiple of 64, N of 32)",
+            p->T, p->K, p->N);
+    }
+    if (p->epilogue != TRTAMD_LINEAR_RAW_INT32 && (p->alpha == nullptr || p->beta == nullptr))
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "int8_linear: alpha and beta are required by this epilogue");
+    }
+    bool const wideOut = p->epilogue == TRTAMD_LINEAR_RAW_INT32 || p->epilogue == TRTAMD_LINEAR_AFFINE_FP16;
+    if (wideOut && p->out_interleaved)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "int8_linear: INT32 and FP16 outputs are linear only");
+    }
+    if ((int64_t) p->T * p->K >= (int64_t) 1 << 31 || (int64_t) p->N * p->K >= (int64_t) 1 << 31)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "int8_linear: operand of 2 GiB or more");
+    }
+    if (!aligned16(p->a) || !aligned16(p->w) || !aligned16(p->out) || (p->alpha && !aligned16(p->alpha))
+        || (p->beta && !aligned16(p->beta)))
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "int8_linear: pointers must be 16-byte aligned");
+    }
+    if (p->T == 0)
+    {
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    LinearArgs a{p->a, p->w, p->alpha, p->beta, p->out, p->T, p->K, p->N, p->out_scale};
+    bool const ilOut = p->out_interleaved != 0;
+    hipStream_t const st = as_stream(stream);
+    if (p->w_interleaved)
+    {
+        return p->a_interleaved ? launch_out<true, true>(st, a, p->epilogue, ilOut)
+                                : launch_out<true, false>(st, a, p->epilogue, ilOut);
+    }
+    return p->a_interleaved ? launch_out<false, true>(st, a, p->epilogue, ilOut)
+                            : launch_out<false, false>(st, a, p->epilogue, ilOut);
+}

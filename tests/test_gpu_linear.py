@@ -1,0 +1,147 @@
+"""INT8 linear layer on the GPU against the CPU oracle, through the C-ABI.
+
+Bar: INT32 accumulators bit-exact; requantised INT8 within 1 LSB (the affine epilogue is the same
+single fmaf on both sides and is expected to agree exactly; the GELU epilogue evaluates erf by a
+rational approximation on the GPU and in binary64 in the oracle); FP16 output within the
+floating-point tolerance.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_fp_close, assert_int8_close, dev, dev_empty, host, rng
+from tensorrt_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+def interleave(x):
+    """[T, C] -> [C/32, T, 32]"""
+    T, Cc = x.shape
+    return np.ascontiguousarray(x.reshape(T, Cc // 32, 32).transpose(1, 0, 2))
+
+
+def run_gpu(a, w, alpha, beta, epilogue, out_scale=1.0, a_il=False, out_il=False, w_il=False):
+    import torch
+    api = capi.api()
+    N, K = w.shape
+    T = a.shape[0]
+    da = dev(interleave(a) if a_il else a)
+    dw = dev(interleave(w) if w_il else w)
+    dal = dev(alpha) if alpha is not None else None
+    dbe = dev(beta) if beta is not None else None
+    if epilogue == capi.LINEAR_RAW_INT32:
+        out = dev_empty((T, N), np.int32, fill=-7)
+    elif epilogue == capi.LINEAR_AFFINE_FP16:
+        out = dev_empty((T, N), np.float16, fill=-7)
+    else:
+        out = dev_empty((N // 32, T, 32) if out_il else (T, N), np.int8, fill=-7)
+    p = capi.Int8LinearParams()
+    p.a, p.w, p.out = da.data_ptr(), dw.data_ptr(), out.data_ptr()
+    p.alpha = dal.data_ptr() if dal is not None else None
+    p.beta = dbe.data_ptr() if dbe is not None else None
+    p.T, p.K, p.N = T, K, N
+    p.a_interleaved, p.out_interleaved, p.epilogue, p.out_scale = int(a_il), int(out_il), epilogue, out_scale
+    p.w_interleaved = int(w_il)
+    api.check(api.int8_linear(torch.cuda.current_stream().cuda_stream, C.byref(p)))
+    torch.cuda.synchronize()
+    return host(out)
+
+
+def problem(seed, T, K, N, full_range=False):
+    r = rng(seed)
+    if full_range:
+        a = r.integers(-128, 128, (T, K)).astype(np.int8)
+        w = r.integers(-128, 128, (N, K)).astype(np.int8)
+    else:
+        a = np.clip(np.rint(r.standard_normal((T, K)) * 30), -127, 127).astype(np.int8)
+        w = np.clip(np.rint(r.standard_normal((N, K)) * 30), -127, 127).astype(np.int8)
+    # scales that put the affine result in the INT8 range with some saturation
+    sd = 30.0 * 30.0 * np.sqrt(K) * (4.0 if full_range else 1.0)
+    alpha = (r.uniform(0.5, 1.5, N) * 50.0 / sd).astype(np.float32)
+    beta = r.uniform(-20, 20, N).astype(np.float32)
+    return a, w, alpha, beta
+
+
+SHAPES = [(1, 64, 32), (17, 64, 32), (300, 128, 96), (256, 1024, 256), (1000, 256, 544), (519, 1024, 1024),
+          (2100, 192, 3072)]
+
+
+@pytest.mark.parametrize("T,K,N", SHAPES)
+@pytest.mark.parametrize("a_il,w_il", [(False, False), (True, True), (True, False), (False, True)])
+def test_accumulators_bit_exact(T, K, N, a_il, w_il):
+    a, w, _, _ = problem(11 + T, T, K, N, full_range=True)
+    # the extreme corner: -128 * -128 summed over K
+    a[0, :] = -128
+    w[0, :] = -128
+    got = run_gpu(a, w, None, None, capi.LINEAR_RAW_INT32, a_il=a_il, w_il=w_il)
+    ref = oracle.int8_linear(a, w, epilogue=oracle.LINEAR_RAW_INT32)
+    assert np.array_equal(got, ref)
+    assert got[0, 0] == 16384 * K
+
+
+@pytest.mark.parametrize("T,K,N", SHAPES)
+@pytest.mark.parametrize("a_il,out_il", [(False, False), (True, True), (False, True), (True, False)])
+def test_affine_int8(T, K, N, a_il, out_il):
+    a, w, alpha, beta = problem(23 + T, T, K, N)
+    got = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=a_il, out_il=out_il, w_il=a_il)
+    ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE, out_interleaved=out_il)
+    assert (np.abs(ref.astype(int)) == 127).any() or (ref == -128).any(), "inputs should exercise saturation"
+    assert_int8_close(got, ref, what="affine", max_frac_off=1e-3)
+
+
+@pytest.mark.parametrize("T,K,N", [(17, 64, 32), (519, 1024, 1024), (700, 1024, 4096)])
+@pytest.mark.parametrize("il", [False, True])
+def test_gelu_int8(T, K, N, il):
+    a, w, alpha, beta = problem(37 + T, T, K, N)
+    alpha = (alpha * 0.06).astype(np.float32)   # pre-activations of a few units either side of zero
+    beta = (beta * 0.02).astype(np.float32)
+    q = np.float32(127.0 / 4.0)
+    got = run_gpu(a, w, alpha, beta, capi.LINEAR_GELU, out_scale=float(q), a_il=il, out_il=il, w_il=il)
+    ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_GELU, out_scale=float(q), out_interleaved=il)
+    assert ref.max() > 60 and ref.min() < 0
+    assert_int8_close(got, ref, what="gelu", max_frac_off=2e-3)
+
+
+@pytest.mark.parametrize("T,K,N", [(33, 64, 64), (519, 1024, 1024)])
+def test_affine_fp16(T, K, N):
+    a, w, alpha, beta = problem(41 + T, T, K, N)
+    got = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE_FP16, a_il=True, w_il=True)
+    ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE_FP16)
+    assert_fp_close(got, ref, what="fp16 output")
+
+
+def test_output_untouched_beyond_the_problem():
+    """Rows beyond T and the bytes of neighbouring allocations are never written."""
+    import torch
+    api = capi.api()
+    T, K, N = 130, 128, 96
+    a, w, alpha, beta = problem(5, T, K, N)
+    da, dw, dal, dbe = dev(a), dev(w), dev(alpha), dev(beta)
+    out = dev_empty((T + 64, N), np.int8, fill=55)
+    p = capi.Int8LinearParams()
+    p.a, p.w, p.alpha, p.beta, p.out = da.data_ptr(), dw.data_ptr(), dal.data_ptr(), dbe.data_ptr(), out.data_ptr()
+    p.T, p.K, p.N, p.epilogue = T, K, N, capi.LINEAR_AFFINE
+    api.check(api.int8_linear(torch.cuda.current_stream().cuda_stream, C.byref(p)))
+    torch.cuda.synchronize()
+    got = host(out)
+    assert (got[T:] == 55).all()
+    assert_int8_close(got[:T], oracle.int8_linear(a, w, alpha, beta), what="affine")
+
+
+def test_bad_arguments_are_refused():
+    api = capi.api()
+    p = capi.Int8LinearParams()
+    assert api.int8_linear(None, C.byref(p)) != 0
+    a, w, alpha, beta = problem(1, 16, 64, 32)
+    da, dw, dal, dbe = dev(a), dev(w), dev(alpha), dev(beta)
+    out = dev_empty((16, 32), np.int8)
+    p.a, p.w, p.alpha, p.beta, p.out = da.data_ptr(), dw.data_ptr(), dal.data_ptr(), dbe.data_ptr(), out.data_ptr()
+    for T, K, N in [(16, 48, 32), (16, 64, 40), (-1, 64, 32)]:
+        p.T, p.K, p.N = T, K, N
+        assert api.int8_linear(None, C.byref(p)) != 0
+        assert "int8_linear" in api.last_error_str()
+    p.T, p.K, p.N, p.epilogue, p.out_interleaved = 16, 64, 32, capi.LINEAR_RAW_INT32, 1
+    assert api.int8_linear(None, C.byref(p)) != 0

@@ -36,6 +36,14 @@ def test_kernel_header_symbols_exported(lib):
     assert sorted(capi.HEADER_SYMBOLS) == names
 
 
+def test_encoder_ops_header_symbols_exported(lib):
+    names = _declared("trtamd_encoder_ops.h", "TRTAMD_API")
+    assert names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in trtamd_encoder_ops.h but not exported"
+    assert sorted(capi.ENCODER_OPS_SYMBOLS) == names
+
+
 def test_plugin_c_header_symbols_exported(lib):
     from tensorrt_amd import plugin
     names = _declared("trtamd_plugin_c.h", "TRTAMD_PLUGIN_API")

@@ -478,3 +478,93 @@ def test_int8_layernorm_all_byte_pairs():
         want = np.clip(np.rint(0.5 * x.astype(np.float64) + 0.25 * s.astype(np.float64)), lo, 127)
         # .5 ties: 0.5*a + 0.25*b is exact in binary16/32, so round-half-even decides identically
         assert np.array_equal(oracle.deinterleave(pre, total, ld), want.astype(np.int8))
+
+
+# ---- INT8 linear layer ---------------------------------------------------------------------------
+
+def _interleave(x):
+    T, Cc = x.shape
+    return np.ascontiguousarray(x.reshape(T, Cc // 32, 32).transpose(1, 0, 2))
+
+
+def test_int8_linear_accumulators_against_int64_matmul():
+    r = rng(3)
+    T, K, N = 37, 192, 96
+    a = r.integers(-128, 128, (T, K)).astype(np.int8)
+    w = r.integers(-128, 128, (N, K)).astype(np.int8)
+    want = a.astype(np.int64) @ w.astype(np.int64).T        # a transposed operand or a dropped row fails here
+    got = oracle.int8_linear(a, w, epilogue=oracle.LINEAR_RAW_INT32)
+    assert np.array_equal(got.astype(np.int64), want)
+    # the interleaved activation layout is only a permutation of the same bytes
+    got_il = oracle.int8_linear(_interleave(a), w, epilogue=oracle.LINEAR_RAW_INT32, a_interleaved=True)
+    assert np.array_equal(got_il, got)
+    # extreme corner: -128 * -128 * K fits INT32 for every K the layers use
+    a[:] = -128
+    w[:] = -128
+    assert (oracle.int8_linear(a, w, epilogue=oracle.LINEAR_RAW_INT32) == 16384 * K).all()
+
+
+def test_int8_linear_identity_weights_pass_the_input_through():
+    r = rng(4)
+    T, K = 20, 64
+    a = r.integers(-128, 128, (T, K)).astype(np.int8)
+    w = np.eye(K, dtype=np.int8)
+    one, zero = np.ones(K, np.float32), np.zeros(K, np.float32)
+    assert np.array_equal(oracle.int8_linear(a, w, one, zero), a)
+    # output layout: channel n of token t lands at [n/32][t][n%32]
+    out_il = oracle.int8_linear(a, w, one, zero, out_interleaved=True)
+    assert np.array_equal(out_il, _interleave(a))
+    # per-channel scale and offset: channel n is doubled and shifted by n - 32, then saturated
+    alpha = np.full(K, 2, np.float32)
+    beta = (np.arange(K) - 32).astype(np.float32)
+    want = np.clip(2 * a.astype(np.int64) + (np.arange(K) - 32)[None, :], -128, 127)
+    assert np.array_equal(oracle.int8_linear(a, w, alpha, beta).astype(np.int64), want)
+
+
+def test_int8_linear_affine_rounds_half_to_even_after_one_fma():
+    # one weight of 1 picks activation k=0; alpha = 0.5 makes every odd activation a tie
+    K, N = 64, 32
+    a = np.zeros((256, K), np.int8)
+    a[:, 0] = np.arange(-128, 128)
+    w = np.zeros((N, K), np.int8)
+    w[:, 0] = 1
+    got = oracle.int8_linear(a, w, np.full(N, 0.5, np.float32), np.zeros(N, np.float32))[:, 0]
+    half = np.arange(-128, 128) / 2.0
+    want = np.where(np.abs(half - np.trunc(half)) == 0.5, 2 * np.round(half / 2), np.round(half))
+    assert np.array_equal(got.astype(np.float64), want)
+    # fused multiply-add: acc*alpha + beta is rounded once.  With acc = 3, alpha = fl(1/3) and beta = -1 a
+    # separately rounded product is exactly 1 and the result 0; the fused result is 3*fl(1/3) - 1 = 2^-25.
+    a1 = np.zeros((1, K), np.int8)
+    a1[0, 0] = 3
+    al = np.full(N, np.float32(1.0) / np.float32(3.0), np.float32)
+    be = np.full(N, -1.0, np.float32)
+    out16 = oracle.int8_linear(a1, w, al * np.float32(2 ** 20), be * np.float32(2 ** 20),
+                               epilogue=oracle.LINEAR_AFFINE_FP16)
+    # both constants scaled by 2^20 so that the result, 2^-5, is a normal binary16 number
+    assert float(out16[0, 0]) == 2.0 ** -5
+
+
+def test_int8_linear_gelu_against_binary64_erf():
+    from scipy.special import erf
+    K, N = 64, 32
+    vals = np.arange(-128, 128)
+    a = np.zeros((256, K), np.int8)
+    a[:, 0] = vals
+    w = np.zeros((N, K), np.int8)
+    w[:, 0] = 1
+    alpha = np.linspace(0.001, 0.06, N).astype(np.float32)      # pre-activations from -7.7 to 7.6
+    beta = np.linspace(-0.5, 0.5, N).astype(np.float32)
+    q = 127.0 / 8.0
+    got = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_GELU, out_scale=q).astype(np.float64)
+    y = vals[:, None].astype(np.float64) * alpha[None, :].astype(np.float64) + beta[None, :].astype(np.float64)
+    g = 0.5 * y * (1.0 + erf(y / np.sqrt(2.0))) * q
+    assert np.abs(got - np.clip(g, -128, 127)).max() <= 0.5 + 1e-4
+    # GELU facts: zero maps to zero, large positive is the identity, large negative vanishes
+    z = oracle.int8_linear(np.zeros((1, K), np.int8), w, alpha, np.zeros(N, np.float32), oracle.LINEAR_GELU, out_scale=q)
+    assert (z == 0).all()
+    big = oracle.int8_linear(a[255:256], w, np.full(N, 0.05, np.float32), np.zeros(N, np.float32), oracle.LINEAR_GELU,
+                             out_scale=10.0)
+    assert (big == round(127 * 0.05 * 10.0)).all()               # gelu(6.35) = 6.35 to 1e-9
+    neg = oracle.int8_linear(a[0:1], w, np.full(N, 0.05, np.float32), np.zeros(N, np.float32), oracle.LINEAR_GELU,
+                             out_scale=10.0)
+    assert (neg == 0).all()
