@@ -55,6 +55,31 @@ typedef struct trtamd_int8_linear_params
  * (closed source; engine-side placement described in plugin/bertQKVToContextPlugin/README.md:25-30). */
 TRTAMD_API int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_params const* params);
 
+/* ------------------------------------------------------------------------------------------
+ * Reformats either side of the interleaved plugins.  TensorRT inserts these itself when a plugin asks
+ * for TensorFormat::kCHW32 (include/NvInferRuntime.h:1471; the INT8 interleaved plugins do:
+ * plugin/bertQKVToContextPlugin/qkvToContextInt8InterleavedPlugin.cpp:124-127,
+ * plugin/skipLayerNormPlugin/skipLayerNormInt8InterleavedPlugin.cpp supportsFormatCombination); here
+ * they are explicit calls.  "linear" is [T][C] (token-major); "interleaved" is [C/32][T][32], the
+ * memory image of a [1,C,T,1] kCHW32 tensor.  C % 32 == 0.
+ * ------------------------------------------------------------------------------------------ */
+
+/* Pure layout change of INT8 data (also used once per weight matrix: [N][K] -> [K/32][N][32]). */
+TRTAMD_API int trtamd_int8_linear_to_interleaved(trtamd_stream_t stream, int32_t T, int32_t C, int8_t const* in,
+    int8_t* out);
+TRTAMD_API int trtamd_int8_interleaved_to_linear(trtamd_stream_t stream, int32_t T, int32_t C, int8_t const* in,
+    int8_t* out);
+
+/* IQuantizeLayer with a per-tensor scale (include/NvInfer.h:5333-5345): out = clamp(round_half_even(in / scale),
+ * -128, 127), fused with the reformat to the interleaved layout. */
+TRTAMD_API int trtamd_quantize_fp16_to_interleaved(trtamd_stream_t stream, int32_t T, int32_t C,
+    trtamd_half_t const* in, float scale, int8_t* out);
+
+/* IDequantizeLayer with a per-tensor scale (include/NvInfer.h:5493-5500): out = binary16(in * scale), fused with
+ * the reformat back to the linear layout. */
+TRTAMD_API int trtamd_dequantize_interleaved_to_fp16(trtamd_stream_t stream, int32_t T, int32_t C, int8_t const* in,
+    float scale, trtamd_half_t* out);
+
 #ifdef __cplusplus
 }
 #endif

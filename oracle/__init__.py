@@ -334,3 +334,21 @@ def int8_linear(a, w, alpha=None, beta=None, epilogue=LINEAR_AFFINE, out_scale=1
     if rc != 0:
         raise ValueError("orc_int8_linear rejected its arguments")
     return out
+
+
+def quantize_f16_interleave(x, scale):
+    """x: float16 [T,C]; returns int8 [C/32,T,32] = clamp(rne(x / scale), -128, 127)."""
+    x = _c(x, np.float16)
+    T, Cc = x.shape
+    out = np.zeros((Cc // 32, T, 32), np.int8)
+    lib().orc_quantize_f16_interleave(_p(x), C.c_float(scale), _p(out), C.c_int64(T), C.c_int(Cc))
+    return out
+
+
+def dequantize_deinterleave_f16(q, scale):
+    """q: int8 [C/32,T,32]; returns float16 [T,C] = binary16(q * scale)."""
+    q = _c(q, np.int8)
+    nslab, T, _ = q.shape
+    out = np.zeros((T, nslab * 32), np.float16)
+    lib().orc_dequantize_deinterleave_f16(_p(q), C.c_float(scale), _p(out), C.c_int64(T), C.c_int(nslab * 32))
+    return out

@@ -1161,3 +1161,29 @@ ORC_API int orc_int8_linear(int64_t T, int K, int N, int8_t const* a, int aInter
     }
     return 0;
 }
+
+/* IQuantizeLayer / IDequantizeLayer with a per-tensor scale, fused with the kCHW32 reformat that
+ * TensorRT inserts around the interleaved plugins (include/NvInfer.h:5333-5345, 5493-5500):
+ *   q = clamp(round_half_even(x / scale), -128, 127)       x = binary16(q * scale)
+ * x is binary16 [T][C]; q is INT8 [C/32][T][32]. */
+ORC_API void orc_quantize_f16_interleave(uint16_t const* x, float scale, int8_t* q, int64_t T, int C)
+{
+    for (int64_t t = 0; t < T; ++t)
+    {
+        for (int c = 0; c < C; ++c)
+        {
+            q[il_index(c, t, T)] = sat8_rne(h2f(x[t * C + c]) / scale);
+        }
+    }
+}
+
+ORC_API void orc_dequantize_deinterleave_f16(int8_t const* q, float scale, uint16_t* x, int64_t T, int C)
+{
+    for (int64_t t = 0; t < T; ++t)
+    {
+        for (int c = 0; c < C; ++c)
+        {
+            x[t * C + c] = d2h((double) ((float) q[il_index(c, t, T)] * scale));
+        }
+    }
+}

@@ -568,3 +568,20 @@ def test_int8_linear_gelu_against_binary64_erf():
     neg = oracle.int8_linear(a[0:1], w, np.full(N, 0.05, np.float32), np.zeros(N, np.float32), oracle.LINEAR_GELU,
                              out_scale=10.0)
     assert (neg == 0).all()
+
+
+def test_quantize_dequantize_reformat_closed_form():
+    r = rng(6)
+    T, Cc = 45, 96
+    x = (r.standard_normal((T, Cc)) * 3).astype(np.float16)
+    x[0, :8] = [0.5, 1.5, 2.5, -0.5, -1.5, 1000, -1000, 0]       # ties go to even, range saturates
+    q = oracle.quantize_f16_interleave(x, 1.0)
+    assert list(q[0, 0, :8]) == [0, 2, 2, 0, -2, 127, -128, 0]
+    scale = np.float32(0.037)
+    q = oracle.quantize_f16_interleave(x, float(scale))
+    want = np.clip(np.rint((x.astype(np.float32) / scale).astype(np.float32)), -128, 127).astype(np.int8)
+    assert np.array_equal(q, _interleave(want))
+    back = oracle.dequantize_deinterleave_f16(q, float(scale))
+    assert np.array_equal(back, (want.astype(np.float32) * scale).astype(np.float16))
+    # quantise(dequantise(q)) is the identity when no value saturates the binary16 mantissa (|q| <= 128)
+    assert np.array_equal(oracle.quantize_f16_interleave(back, float(scale)), q)
