@@ -51,6 +51,8 @@ struct LinearArgs
     void* out;
     int T, K, N;
     float qOut;
+    int mainTiles; // workgroups that own a 256 x 256 tile
+    int tokMain;   // rows of 256 tokens they cover
 };
 
 // 0.5 * erfc(|y| / sqrt(2)) by the rational-exponential form of Abramowitz & Stegun 7.1.26
@@ -93,8 +95,10 @@ __device__ inline int frag_offset(int row, int half)
     return row * 32 + ((half ^ ((row >> 3) & 1)) << 4);
 }
 
+// One output tile of BM = WM*MT*32 channels x BN = WN*NT*32 tokens at (n0, t0), by the whole workgroup.
 template <int WM, int WN, int MT, int NT, bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
-__global__ __launch_bounds__(64 * WM * WN) void int8_linear_kernel(LinearArgs const p)
+__device__ __forceinline__ void linear_tile(
+    LinearArgs const& p, int const n0, int const t0, uint8_t* __restrict__ lds, float* sAlpha, float* sBeta)
 {
     constexpr int NWAVES = WM * WN;
     constexpr int BM = WM * MT * 32;    // output channels per workgroup
@@ -106,23 +110,12 @@ __global__ __launch_bounds__(64 * WM * WN) void int8_linear_kernel(LinearArgs co
     constexpr int LB = BF / NWAVES;
     constexpr int STAGE = (AF + BF) * 1024;
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * STAGE];
-    __shared__ __attribute__((aligned(16))) float sAlpha[BM];
-    __shared__ __attribute__((aligned(16))) float sBeta[BM];
-
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const wm = wave / WN;
     int const wn = wave % WN;
     int const col32 = lane & 31;
     int const hi = lane >> 5;
-
-    // channel tiles vary fastest, so the workgroups resident on one XCD share a few token tiles
-    // (read from HBM once into that XCD's L2) and sweep all the weights
-    uint32_t const nbm = (uint32_t) ((p.N + BM - 1) / BM);
-    uint32_t const tile = xcd_remap(blockIdx.x, gridDim.x);
-    int const n0 = (int) (tile % nbm) * BM;
-    int const t0 = (int) (tile / nbm) * BN;
 
     // A load unit is 1 KB that one wave fetches with one 16-byte load per lane, consecutive lanes
     // reading consecutive memory.  Interleaved operand [K/32][R][32]: unit (rb, ks) is the 32 rows of
@@ -369,36 +362,67 @@ __global__ __launch_bounds__(64 * WM * WN) void int8_linear_kernel(LinearArgs co
     }
 }
 
-template <int WM, int WN, int MT, int NT, bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
-int launch_tile(hipStream_t stream, LinearArgs const& a)
+// Tokens [0, 256*tokMain) are cut into 256 x 256 tiles (workgroups 0 .. mainTiles-1); what is left, which
+// would otherwise be a last round of big tiles on a fraction of the CUs, is cut into 128 x 128 tiles that
+// spread over all of them.
+constexpr int kBig = 256;
+constexpr int kSmall = 128;
+
+template <bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
+__global__ __launch_bounds__(512) void int8_linear_kernel(LinearArgs const p)
 {
-    constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
-    uint32_t const grid = (uint32_t) ceil_div(a.N, BM) * (uint32_t) ceil_div(a.T, BN);
-    hipLaunchKernelGGL((int8_linear_kernel<WM, WN, MT, NT, IL_W, IL_IN, IL_OUT, EPI>), dim3(grid), dim3(64 * WM * WN),
-        0, stream, a);
-    return check_launch("int8_linear_kernel");
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * 2 * (kBig / 32) * 2 * 1024];
+    __shared__ __attribute__((aligned(16))) float sAlpha[kBig];
+    __shared__ __attribute__((aligned(16))) float sBeta[kBig];
+    if ((int) blockIdx.x < p.mainTiles)
+    {
+        // channel tiles vary fastest, so the workgroups resident on one XCD share a few token tiles
+        // (read from HBM once into that XCD's L2) and sweep all the weights
+        uint32_t const nbm = (uint32_t) ((p.N + kBig - 1) / kBig);
+        uint32_t const tile = xcd_remap(blockIdx.x, (uint32_t) p.mainTiles);
+        linear_tile<2, 4, 4, 2, IL_W, IL_IN, IL_OUT, EPI>(
+            p, (int) (tile % nbm) * kBig, (int) (tile / nbm) * kBig, lds, sAlpha, sBeta);
+    }
+    else
+    {
+        uint32_t const nbm = (uint32_t) ((p.N + kSmall - 1) / kSmall);
+        uint32_t const tile = blockIdx.x - (uint32_t) p.mainTiles;
+        linear_tile<2, 4, 2, 1, IL_W, IL_IN, IL_OUT, EPI>(
+            p, (int) (tile % nbm) * kSmall, p.tokMain * kBig + (int) (tile / nbm) * kSmall, lds, sAlpha, sBeta);
+    }
+}
+
+int num_cus()
+{
+    static int const n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess
+            || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        {
+            cus = 256;
+        }
+        return cus;
+    }();
+    return n;
 }
 
 template <bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
-int launch_shape(hipStream_t stream, LinearArgs const& a)
+int launch_shape(hipStream_t stream, LinearArgs a)
 {
-    static int const forced = [] {
-        char const* e = getenv("TRTAMD_LINEAR_TILE");
-        return e ? atoi(e) : -1;
-    }();
-    // large problems: 256 channels x 256 tokens per workgroup; small ones: 128 x 128 so that the
-    // launch still has a workgroup for every CU
-    int64_t const big = (int64_t) ceil_div(a.N, 256) * ceil_div(a.T, 256);
-    int const choice = forced >= 0 ? forced : (big >= 256 ? 0 : 1);
-    switch (choice)
+    // big tiles for as many whole token-tile rows as fit in full rounds of one workgroup per CU
+    int const nbmBig = ceil_div(a.N, kBig);
+    int64_t const bigTiles = (int64_t) nbmBig * (a.T / kBig);
+    int const cus = num_cus();
+    a.tokMain = (int) ((bigTiles / cus) * cus / nbmBig);
+    a.mainTiles = a.tokMain * nbmBig;
+    int const restTokens = a.T - a.tokMain * kBig;
+    int64_t const grid = (int64_t) a.mainTiles + (int64_t) ceil_div(a.N, kSmall) * ceil_div(restTokens, kSmall);
+    if (grid >= (int64_t) 1 << 31)
     {
-    case 0: return launch_tile<2, 4, 4, 2, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
-    case 1: return launch_tile<2, 2, 2, 2, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
-    case 2: return launch_tile<4, 2, 2, 4, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
-    case 3: return launch_tile<2, 2, 4, 2, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
-    case 4: return launch_tile<2, 2, 2, 4, IL_W, IL_IN, IL_OUT, EPI>(stream, a);
-    default: return set_error(TRTAMD_STATUS_BAD_PARAM, "TRTAMD_LINEAR_TILE=%d is not a tile configuration", choice);
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "int8_linear: too many tiles");
     }
+    hipLaunchKernelGGL((int8_linear_kernel<IL_W, IL_IN, IL_OUT, EPI>), dim3((uint32_t) grid), dim3(512), 0, stream, a);
+    return check_launch("int8_linear_kernel");
 }
 
 template <bool IL_W, bool IL_IN>
@@ -455,7 +479,7 @@ extern "C" int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_par
     {
         return TRTAMD_STATUS_SUCCESS;
     }
-    LinearArgs a{p->a, p->w, p->alpha, p->beta, p->out, p->T, p->K, p->N, p->out_scale};
+    LinearArgs a{p->a, p->w, p->alpha, p->beta, p->out, p->T, p->K, p->N, p->out_scale, 0, 0};
     bool const ilOut = p->out_interleaved != 0;
     hipStream_t const st = as_stream(stream);
     if (p->w_interleaved)

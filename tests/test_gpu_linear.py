@@ -113,6 +113,21 @@ def test_affine_fp16(T, K, N):
     assert_fp_close(got, ref, what="fp16 output")
 
 
+@pytest.mark.parametrize("T,K,N", [(8229, 128, 3072), (16500, 64, 1024), (70000, 64, 256)])
+def test_large_problems_mix_both_tile_sizes(T, K, N):
+    """Enough 256 x 256 tiles for whole rounds of the chip, plus a remainder in 128 x 128 tiles."""
+    a, w, alpha, beta = problem(51 + T, T, K, N, full_range=True)
+    got = run_gpu(a, w, None, None, capi.LINEAR_RAW_INT32, a_il=True, w_il=True)
+    ref = oracle.int8_linear(a, w, epilogue=oracle.LINEAR_RAW_INT32)
+    assert np.array_equal(got, ref)
+    got8 = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=True, w_il=True, out_il=True)
+    ref8 = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE, out_interleaved=True)
+    assert_int8_close(got8, ref8, what="affine", max_frac_off=1e-3)
+    got_lin = run_gpu(a, w, alpha, beta, capi.LINEAR_GELU, out_scale=0.5)
+    ref_lin = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_GELU, out_scale=0.5)
+    assert_int8_close(got_lin, ref_lin, what="gelu, linear layouts", max_frac_off=2e-3)
+
+
 def test_output_untouched_beyond_the_problem():
     """Rows beyond T and the bytes of neighbouring allocations are never written."""
     import torch
