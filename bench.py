@@ -207,7 +207,7 @@ def run_encoder(args, api, torch):
             "layers": cfg.layers, "tokens": T, "lengths": f"uniform[128,{args.seqlen}] seed {args.seed}",
         },
         "roofline": {
-            "kernel": "int8_linear_kernel<true,true,true,GELU> (feed-forward 1)",
+            "kernel": "int8_linear_persistent_kernel<true,true,true,GELU> (feed-forward 1)",
             "bound": "mfma",
             "achieved": table[dom]["TOP/s"],
             "peak": PEAK_INT8_OPS / 1e12,

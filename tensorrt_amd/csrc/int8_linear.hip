@@ -33,6 +33,7 @@ namespace
 
 constexpr float kRoundMagic = 12582912.f; // 1.5 * 2^23: adding it rounds to nearest even
 constexpr int kRoundMagicBits = 0x4B400000;
+constexpr int kBigTile = 256; // channels and tokens of the large workgroup tile
 
 enum Epilogue
 {
@@ -54,6 +55,7 @@ struct LinearArgs
     int mainTiles; // workgroups that own a 256 x 256 tile
     int tokMain;   // rows of 256 tokens they cover
     int panel;     // channel tiles per panel of the tile numbering (divides the number of channel tiles)
+    int persist;   // persistent kernel: workgroups that loop over the 256 x 256 tiles
 };
 
 // gelu(y) = y * Phi(y) = max(y, 0) - |y| * Phi(-|y|).  log2(Phi(-a)) is smooth and nearly quadratic, so
@@ -98,6 +100,114 @@ __device__ inline uint32_t low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint
 __device__ inline int frag_offset(int row, int half)
 {
     return row * 32 + ((half ^ ((row >> 3) & 1)) << 4);
+}
+
+// Epilogue of one workgroup tile.  Accumulator register v of a 32x32 tile is token l%32, channel
+// 8*(v/4) + 4*(l/32) + v%4: four groups of four consecutive channels.  For the INT8 outputs the two lanes
+// that share a token trade two packed dwords (v_permlane32_swap), after which lane l holds the 16
+// consecutive channels 16*(l/32)..+15 and stores them with one 16-byte write.
+template <int WM, int WN, int MT, int NT, bool IL_OUT, int EPI>
+__device__ __forceinline__ void store_tile(LinearArgs const& p, i32x16 const (&acc)[MT][NT], int const n0, int const t0,
+    float const* sAlpha, float const* sBeta)
+{
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const wm = wave / WN;
+    int const wn = wave % WN;
+    int const col32 = lane & 31;
+    int const hi = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+    {
+        int const cl = (wm * MT + i) * 32; // wave-uniform, and so is the guard: N is a multiple of 32
+        if (n0 + cl >= p.N)
+        {
+            break;
+        }
+        f32x4 al[4], be[4];
+        if constexpr (EPI != kRAW)
+        {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + cl + 8 * g + 4 * hi);
+                be[g] = *reinterpret_cast<f32x4 const*>(sBeta + cl + 8 * g + 4 * hi);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+        {
+            int const t = t0 + (wn * NT + j) * 32 + col32;
+            bool const live = t < p.T;
+            if constexpr (EPI == kRAW)
+            {
+                if (live)
+                {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        i32x4 const v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                            acc[i][j][4 * g + 3]};
+                        *reinterpret_cast<i32x4*>(
+                            static_cast<int32_t*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
+                            = v;
+                    }
+                }
+            }
+            else if constexpr (EPI == kHALF)
+            {
+                if (live)
+                {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        f16x4 h;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            h[e] = (f16) fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
+                        }
+                        *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
+                            = h;
+                    }
+                }
+            }
+            else
+            {
+                int d[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    uint32_t b[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        float y = fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
+                        if constexpr (EPI == kGELU)
+                        {
+                            // one rounding of gelu * scale + 1.5*2^23: the sum's low bits are the integer
+                            b[e] = clamp_sat8_bits(fmaf(gelu_erf(y), p.qOut, kRoundMagic));
+                        }
+                        else
+                        {
+                            b[e] = round_sat8_bits(y);
+                        }
+                    }
+                    d[g] = (int) low_bytes(b[0], b[1], b[2], b[3]);
+                }
+                // lanes l < 32 hold channels [0-3][8-11][16-19][24-27], lanes l+32 the gaps
+                auto const s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                auto const s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+                i32x4 const packed = {(int) s02[0], (int) s02[1], (int) s13[0], (int) s13[1]};
+                if (live)
+                {
+                    int const c = n0 + cl + 16 * hi;
+                    size_t const o = IL_OUT ? ((size_t) (c >> 5) * p.T + t) * 32 + (c & 31) : (size_t) t * p.N + c;
+                    *reinterpret_cast<i32x4*>(static_cast<int8_t*>(p.out) + o) = packed;
+                }
+            }
+        }
+    }
 }
 
 // One output tile of BM = WM*MT*32 channels x BN = WN*NT*32 tokens at (n0, t0), by the whole workgroup.
@@ -272,101 +382,212 @@ __device__ __forceinline__ void linear_tile(
         multiply(0);
     }
 
-    // ---- epilogue -------------------------------------------------------------------------------
-    // Accumulator register v of a 32x32 tile is token l%32, channel 8*(v/4) + 4*(l/32) + v%4: four
-    // groups of four consecutive channels.  For the INT8 outputs the two lanes that share a token
-    // trade two packed dwords (v_permlane32_swap), after which lane l holds the 16 consecutive
-    // channels 16*(l/32)..+15 and stores them with one 16-byte write.
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-    {
-        int const cl = (wm * MT + i) * 32; // wave-uniform, and so is the guard: N is a multiple of 32
-        if (n0 + cl >= p.N)
-        {
-            break;
-        }
-        f32x4 al[4], be[4];
-        if constexpr (EPI != kRAW)
-        {
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
+    store_tile<WM, WN, MT, NT, IL_OUT, EPI>(p, acc, n0, t0, sAlpha, sBeta);
+}
+
+// A run of `count` tiles by one persistent workgroup, K % 128 == 0.  The stage pipeline does not drain
+// between tiles: the last two stages of a tile already fetch the first two stages of the next one, the
+// epilogue runs while those loads are in flight, and the next tile's scale/offset vectors are picked up at
+// the start of the current one.  `origin(j, n0, t0)` gives the j-th tile's corner.
+template <int WM, int WN, int MT, int NT, bool IL_W, bool IL_IN, bool IL_OUT, int EPI, typename Origin>
+__device__ __forceinline__ void linear_tile_run(
+    LinearArgs const& p, int const count, Origin origin, uint8_t* __restrict__ lds, float* sScale)
+{
+    constexpr int NWAVES = WM * WN;
+    constexpr int BM = WM * MT * 32;
+    constexpr int BN = WN * NT * 32;
+    constexpr int AF = (BM / 32) * 2;
+    constexpr int BF = (BN / 32) * 2;
+    static_assert(AF % NWAVES == 0 && BF % NWAVES == 0, "load units divide evenly among the waves");
+    static_assert((BM & (BM - 1)) == 0 && BM <= kBigTile, "scale staging");
+    constexpr int LA = AF / NWAVES;
+    constexpr int LB = BF / NWAVES;
+    constexpr int STAGE = (AF + BF) * 1024;
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const wm = wave / WN;
+    int const wn = wave % WN;
+
+    int ldsA[LA], ldsB[LB];
+    auto address = [&](int n0, int t0, uint32_t(&oa)[LA], uint32_t(&ob)[LB]) {
+        auto unit = [&](bool interleaved, int u, int row0, int R, uint32_t& gOff, int& lOff) {
+            int const rb = u >> 1, sel = u & 1;
+            if (interleaved)
             {
-                al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + cl + 8 * g + 4 * hi);
-                be[g] = *reinterpret_cast<f32x4 const*>(sBeta + cl + 8 * g + 4 * hi);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-        {
-            int const t = t0 + (wn * NT + j) * 32 + col32;
-            bool const live = t < p.T;
-            if constexpr (EPI == kRAW)
-            {
-                if (live)
-                {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                    {
-                        i32x4 const v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                            acc[i][j][4 * g + 3]};
-                        *reinterpret_cast<i32x4*>(
-                            static_cast<int32_t*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
-                            = v;
-                    }
-                }
-            }
-            else if constexpr (EPI == kHALF)
-            {
-                if (live)
-                {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                    {
-                        f16x4 h;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                        {
-                            h[e] = (f16) fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
-                        }
-                        *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
-                            = h;
-                    }
-                }
+                int const r = lane >> 1, c = lane & 1;
+                int const row = min(row0 + rb * 32 + r, R - 1);
+                gOff = ((uint32_t) sel * (uint32_t) R + (uint32_t) row) * 32u + (uint32_t) c * 16u;
+                lOff = (rb * 2 + sel) * 1024 + frag_offset(r, c);
             }
             else
             {
-                int d[4];
+                int const r = sel * 16 + (lane >> 2), c = lane & 3;
+                int const row = min(row0 + rb * 32 + r, R - 1);
+                gOff = (uint32_t) row * (uint32_t) p.K + (uint32_t) c * 16u;
+                lOff = (rb * 2 + (c >> 1)) * 1024 + frag_offset(r, c & 1);
+            }
+        };
 #pragma unroll
-                for (int g = 0; g < 4; ++g)
-                {
-                    uint32_t b[4];
+        for (int q = 0; q < LA; ++q)
+        {
+            unit(IL_W, q * NWAVES + wave, n0, p.N, oa[q], ldsA[q]);
+        }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                    {
-                        float y = fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
-                        if constexpr (EPI == kGELU)
-                        {
-                            // one rounding of gelu * scale + 1.5*2^23: the sum's low bits are the integer
-                            b[e] = clamp_sat8_bits(fmaf(gelu_erf(y), p.qOut, kRoundMagic));
-                        }
-                        else
-                        {
-                            b[e] = round_sat8_bits(y);
-                        }
-                    }
-                    d[g] = (int) low_bytes(b[0], b[1], b[2], b[3]);
-                }
-                // lanes l < 32 hold channels [0-3][8-11][16-19][24-27], lanes l+32 the gaps
-                auto const s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-                auto const s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-                i32x4 const packed = {(int) s02[0], (int) s02[1], (int) s13[0], (int) s13[1]};
-                if (live)
+        for (int q = 0; q < LB; ++q)
+        {
+            unit(IL_IN, q * NWAVES + wave, t0, p.T, ob[q], ldsB[q]);
+            ldsB[q] += AF * 1024;
+        }
+    };
+    uint32_t const stepA = IL_W ? 2u * (uint32_t) p.N * 32u : 64u;
+    uint32_t const stepB = IL_IN ? 2u * (uint32_t) p.T * 32u : 64u;
+
+    i32x4 ga[2][LA], gb[2][LB];
+    auto fetch = [&](auto set, uint32_t const(&oa)[LA], uint32_t const(&ob)[LB], int kt) {
+        constexpr int S = decltype(set)::value;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            ga[S][q] = *reinterpret_cast<i32x4 const*>(p.w + oa[q] + (uint32_t) kt * stepA);
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            gb[S][q] = *reinterpret_cast<i32x4 const*>(p.a + ob[q] + (uint32_t) kt * stepB);
+        }
+    };
+    auto stash = [&](auto set, int buf) {
+        constexpr int S = decltype(set)::value;
+        uint8_t* base = lds + buf * STAGE;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            *reinterpret_cast<i32x4*>(base + ldsA[q]) = ga[S][q];
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            *reinterpret_cast<i32x4*>(base + ldsB[q]) = gb[S][q];
+        }
+    };
+
+    i32x16 acc[MT][NT];
+    int const readOff = frag_offset(lane & 31, lane >> 5);
+    auto multiply = [&](int buf) {
+        uint8_t const* base = lds + buf * STAGE + readOff;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+        {
+            i32x4 fa[MT], fb[NT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+            {
+                fa[i] = *reinterpret_cast<i32x4 const*>(base + ((wm * MT + i) * 2 + ks) * 1024);
+            }
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+            {
+                fb[j] = *reinterpret_cast<i32x4 const*>(base + (AF + (wn * NT + j) * 2 + ks) * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+            {
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
                 {
-                    int const c = n0 + cl + 16 * hi;
-                    size_t const o = IL_OUT ? ((size_t) (c >> 5) * p.T + t) * 32 + (c & 31) : (size_t) t * p.N + c;
-                    *reinterpret_cast<i32x4*>(static_cast<int8_t*>(p.out) + o) = packed;
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
                 }
             }
+        }
+    };
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, 1>;
+
+    // scale/offset vectors: sScale[parity][alpha|beta][channel]; every thread copies channel tid % BM
+    int const ch = threadIdx.x & (BM - 1);
+    auto scales = [&](int parity, int which) { return sScale + (parity * 2 + which) * kBigTile; };
+
+    int n0, t0;
+    origin(0, n0, t0);
+    uint32_t oaC[LA], obC[LB], oaN[LA], obN[LB];
+    address(n0, t0, oaC, obC);
+    if constexpr (EPI != kRAW)
+    {
+        int const n = min(n0 + ch, p.N - 1);
+        scales(0, 0)[ch] = p.alpha[n];
+        scales(0, 1)[ch] = p.beta[n];
+    }
+    int const nk = p.K / 64; // even, >= 2
+    fetch(Set0{}, oaC, obC, 0);
+    fetch(Set1{}, oaC, obC, 1);
+    stash(Set0{}, 0);
+    __syncthreads();
+    for (int j = 0; j < count; ++j)
+    {
+        int n1 = n0, t1 = t0;
+        if (j + 1 < count)
+        {
+            origin(j + 1, n1, t1);
+        }
+        address(n1, t1, oaN, obN);
+        float nextAlpha = 0.f, nextBeta = 0.f;
+        if constexpr (EPI != kRAW)
+        {
+            int const n = min(n1 + ch, p.N - 1);
+            nextAlpha = p.alpha[n];
+            nextBeta = p.beta[n];
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+        {
+#pragma unroll
+            for (int jj = 0; jj < NT; ++jj)
+            {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                {
+                    acc[i][jj][v] = 0;
+                }
+            }
+        }
+        for (int kt = 0; kt + 2 < nk; kt += 2)
+        {
+            fetch(Set0{}, oaC, obC, kt + 2);
+            multiply(0);
+            stash(Set1{}, 1);
+            __syncthreads();
+            fetch(Set1{}, oaC, obC, kt + 3);
+            multiply(1);
+            stash(Set0{}, 0);
+            __syncthreads();
+        }
+        // last two stages of this tile; the loads are the next tile's first two stages
+        fetch(Set0{}, oaN, obN, 0);
+        multiply(0);
+        stash(Set1{}, 1);
+        __syncthreads();
+        fetch(Set1{}, oaN, obN, 1);
+        multiply(1);
+        if constexpr (EPI != kRAW)
+        {
+            scales((j + 1) & 1, 0)[ch] = nextAlpha;
+            scales((j + 1) & 1, 1)[ch] = nextBeta;
+        }
+        store_tile<WM, WN, MT, NT, IL_OUT, EPI>(p, acc, n0, t0, scales(j & 1, 0), scales(j & 1, 1));
+        stash(Set0{}, 0);
+        __syncthreads();
+        n0 = n1;
+        t0 = t1;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            oaC[q] = oaN[q];
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            obC[q] = obN[q];
         }
     }
 }
@@ -374,7 +595,7 @@ __device__ __forceinline__ void linear_tile(
 // Tokens [0, 256*tokMain) are cut into 256 x 256 tiles (workgroups 0 .. mainTiles-1); what is left, which
 // would otherwise be a last round of big tiles on a fraction of the CUs, is cut into 128 x 128 tiles that
 // spread over all of them.
-constexpr int kBig = 256;
+constexpr int kBig = kBigTile;
 constexpr int kSmall = 128;
 
 template <bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
@@ -402,6 +623,38 @@ __global__ __launch_bounds__(512) void int8_linear_kernel(LinearArgs const p)
         uint32_t const tile = blockIdx.x - (uint32_t) p.mainTiles;
         linear_tile<2, 4, 2, 1, IL_W, IL_IN, IL_OUT, EPI>(
             p, (int) (tile % nbm) * kSmall, p.tokMain * kBig + (int) (tile / nbm) * kSmall, lds, sAlpha, sBeta);
+    }
+}
+
+// The same tile plan run by persistent workgroups (K % 128 == 0): workgroups 0 .. persist-1 take the
+// 256 x 256 tiles b, b + persist, ... in the panel numbering, the workgroups after them one 128 x 128 tile each.
+template <bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
+__global__ __launch_bounds__(512) void int8_linear_persistent_kernel(LinearArgs const p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * 2 * (kBig / 32) * 2 * 1024];
+    __shared__ __attribute__((aligned(16))) float sScale[2 * 2 * kBig];
+    if ((int) blockIdx.x < p.persist)
+    {
+        uint32_t const pw = (uint32_t) p.panel;
+        uint32_t const perPanel = (uint32_t) p.tokMain * pw;
+        int const count = (p.mainTiles - (int) blockIdx.x + p.persist - 1) / p.persist;
+        auto origin = [&](int j, int& n0, int& t0) {
+            uint32_t const tile = xcd_remap(blockIdx.x + (uint32_t) j * (uint32_t) p.persist, (uint32_t) p.mainTiles);
+            uint32_t const pan = tile / perPanel, rem = tile % perPanel;
+            n0 = (int) (pan * pw + rem % pw) * kBig;
+            t0 = (int) (rem / pw) * kBig;
+        };
+        linear_tile_run<2, 4, 4, 2, IL_W, IL_IN, IL_OUT, EPI>(p, count, origin, lds, sScale);
+    }
+    else
+    {
+        uint32_t const nbm = (uint32_t) ((p.N + kSmall - 1) / kSmall);
+        uint32_t const tile = blockIdx.x - (uint32_t) p.persist;
+        auto origin = [&](int, int& n0, int& t0) {
+            n0 = (int) (tile % nbm) * kSmall;
+            t0 = p.tokMain * kBig + (int) (tile / nbm) * kSmall;
+        };
+        linear_tile_run<2, 4, 2, 1, IL_W, IL_IN, IL_OUT, EPI>(p, 1, origin, lds, sScale);
     }
 }
 
@@ -445,6 +698,18 @@ int launch_shape(hipStream_t stream, LinearArgs a)
     if (grid >= (int64_t) 1 << 31)
     {
         return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "int8_linear: too many tiles");
+    }
+    static int const persistent = [] {
+        char const* e = getenv("TRTAMD_LINEAR_PERSISTENT");
+        return e ? atoi(e) : 1;
+    }();
+    if (persistent && a.K % 128 == 0)
+    {
+        a.persist = a.mainTiles < cus ? a.mainTiles : cus;
+        int64_t const pgrid = grid - a.mainTiles + a.persist;
+        hipLaunchKernelGGL((int8_linear_persistent_kernel<IL_W, IL_IN, IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0,
+            stream, a);
+        return check_launch("int8_linear_persistent_kernel");
     }
     hipLaunchKernelGGL((int8_linear_kernel<IL_W, IL_IN, IL_OUT, EPI>), dim3((uint32_t) grid), dim3(512), 0, stream, a);
     return check_launch("int8_linear_kernel");
@@ -504,7 +769,7 @@ extern "C" int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_par
     {
         return TRTAMD_STATUS_SUCCESS;
     }
-    LinearArgs a{p->a, p->w, p->alpha, p->beta, p->out, p->T, p->K, p->N, p->out_scale, 0, 0, 1};
+    LinearArgs a{p->a, p->w, p->alpha, p->beta, p->out, p->T, p->K, p->N, p->out_scale, 0, 0, 1, 0};
     bool const ilOut = p->out_interleaved != 0;
     hipStream_t const st = as_stream(stream);
     if (p->w_interleaved)
