@@ -19,6 +19,9 @@
  *   VDimensionExpr, VExprBuilder                                       include/NvInferImpl.h:232-264
  *   IPluginRegistry                                                    include/NvInferRuntimeCommon.h:55-249
  *   initLibNvInferPlugins                                              include/NvInferPlugin.h:29-40
+ *   PluginVersion, PluginFormat, IPluginV2, IPluginV2Ext, IPluginCreator include/NvInferRuntimePlugin.h:54, 94-106,
+ *                                                                      138-460, 473-660, 784-909
+ *   IPluginV2DynamicExt                                                include/NvInferRuntime.h:406-570
  * The stream argument of enqueue() is a hipStream_t (an opaque pointer, like cudaStream_t).
  */
 #ifndef TRTAMD_NVINFER_API_H
@@ -31,6 +34,8 @@
 #define NV_TENSORRT_MINOR 1
 #define NV_TENSORRT_PATCH 0
 #define NV_TENSORRT_BUILD 106
+#define NV_TENSORRT_VERSION_INT(major, minor, patch) ((major) *10000L + (minor) *100L + (patch) *1L)
+#define NV_TENSORRT_VERSION NV_TENSORRT_VERSION_INT(NV_TENSORRT_MAJOR, NV_TENSORRT_MINOR, NV_TENSORRT_PATCH)
 
 #ifndef TENSORRTAPI
 #define TENSORRTAPI __attribute__((visibility("default")))
@@ -542,6 +547,167 @@ public:
 
 private:
     T instance{};
+};
+} // namespace nvinfer1
+
+/* ---- the deprecated IPluginV2 family, kept because the reference still ships "Legacy" versions of the
+ *      three BERT plugins on it (the *Legacy.h / *Legacy.cpp files of the three plugin directories) ------ */
+struct cudnnContext;  /* never dereferenced: attachToContext() receives null on this platform */
+struct cublasContext;
+
+namespace nvinfer1
+{
+using PluginFormat = TensorFormat;
+
+constexpr uint8_t kPLUGIN_VERSION_PYTHON_BIT = 0x40;
+enum class PluginVersion : uint8_t
+{
+    kV2 = 0,
+    kV2_EXT = 1,
+    kV2_IOEXT = 2,
+    kV2_DYNAMICEXT = 3,
+    kV2_DYNAMICEXT_PYTHON = kPLUGIN_VERSION_PYTHON_BIT | 3
+};
+
+class IPluginV2
+{
+public:
+    virtual int32_t getTensorRTVersion() const noexcept
+    {
+        return NV_TENSORRT_VERSION;
+    }
+    virtual AsciiChar const* getPluginType() const noexcept = 0;
+    virtual AsciiChar const* getPluginVersion() const noexcept = 0;
+    virtual int32_t getNbOutputs() const noexcept = 0;
+    virtual Dims getOutputDimensions(int32_t index, Dims const* inputs, int32_t nbInputDims) noexcept = 0;
+    virtual bool supportsFormat(DataType type, PluginFormat format) const noexcept = 0;
+    virtual void configureWithFormat(Dims const* inputDims, int32_t nbInputs, Dims const* outputDims,
+        int32_t nbOutputs, DataType type, PluginFormat format, int32_t maxBatchSize) noexcept = 0;
+    virtual int32_t initialize() noexcept = 0;
+    virtual void terminate() noexcept = 0;
+    virtual size_t getWorkspaceSize(int32_t maxBatchSize) const noexcept = 0;
+    virtual int32_t enqueue(int32_t batchSize, void const* const* inputs, void* const* outputs, void* workspace,
+        hipStream_t stream) noexcept = 0;
+    virtual size_t getSerializationSize() const noexcept = 0;
+    virtual void serialize(void* buffer) const noexcept = 0;
+    virtual void destroy() noexcept = 0;
+    virtual IPluginV2* clone() const noexcept = 0;
+    virtual void setPluginNamespace(AsciiChar const* pluginNamespace) noexcept = 0;
+    virtual AsciiChar const* getPluginNamespace() const noexcept = 0;
+
+    IPluginV2() = default;
+    virtual ~IPluginV2() noexcept = default;
+
+protected:
+    IPluginV2(IPluginV2 const&) = default;
+    IPluginV2(IPluginV2&&) = default;
+    IPluginV2& operator=(IPluginV2 const&) & = default;
+    IPluginV2& operator=(IPluginV2&&) & = default;
+};
+
+class IPluginV2Ext : public IPluginV2
+{
+public:
+    virtual DataType getOutputDataType(int32_t index, DataType const* inputTypes, int32_t nbInputs) const noexcept = 0;
+    virtual void configurePlugin(Dims const* inputDims, int32_t nbInputs, Dims const* outputDims, int32_t nbOutputs,
+        DataType const* inputTypes, DataType const* outputTypes, bool const* inputIsBroadcast,
+        bool const* outputIsBroadcast, PluginFormat floatFormat, int32_t maxBatchSize) noexcept = 0;
+
+    IPluginV2Ext() = default;
+    ~IPluginV2Ext() override = default;
+
+    virtual void attachToContext(cudnnContext*, cublasContext*, IGpuAllocator*) noexcept {}
+    virtual void detachFromContext() noexcept {}
+    IPluginV2Ext* clone() const noexcept override = 0;
+
+protected:
+    IPluginV2Ext(IPluginV2Ext const&) = default;
+    IPluginV2Ext(IPluginV2Ext&&) = default;
+    IPluginV2Ext& operator=(IPluginV2Ext const&) & = default;
+    IPluginV2Ext& operator=(IPluginV2Ext&&) & = default;
+
+    int32_t getTensorRTVersion() const noexcept override
+    {
+        return static_cast<int32_t>((static_cast<uint32_t>(PluginVersion::kV2_EXT) << 24U)
+            | (static_cast<uint32_t>(NV_TENSORRT_VERSION) & 0xFFFFFFU));
+    }
+    void configureWithFormat(Dims const*, int32_t, Dims const*, int32_t, DataType, PluginFormat, int32_t) noexcept override
+    {
+    }
+};
+
+class IPluginV2DynamicExt : public IPluginV2Ext
+{
+public:
+    IPluginV2DynamicExt* clone() const noexcept override = 0;
+    virtual DimsExprs getOutputDimensions(
+        int32_t outputIndex, DimsExprs const* inputs, int32_t nbInputs, IExprBuilder& exprBuilder) noexcept = 0;
+    static constexpr int32_t kFORMAT_COMBINATION_LIMIT = 100;
+    virtual bool supportsFormatCombination(
+        int32_t pos, PluginTensorDesc const* inOut, int32_t nbInputs, int32_t nbOutputs) noexcept = 0;
+    virtual void configurePlugin(DynamicPluginTensorDesc const* in, int32_t nbInputs,
+        DynamicPluginTensorDesc const* out, int32_t nbOutputs) noexcept = 0;
+    virtual size_t getWorkspaceSize(PluginTensorDesc const* inputs, int32_t nbInputs, PluginTensorDesc const* outputs,
+        int32_t nbOutputs) const noexcept = 0;
+    virtual int32_t enqueue(PluginTensorDesc const* inputDesc, PluginTensorDesc const* outputDesc,
+        void const* const* inputs, void* const* outputs, void* workspace, hipStream_t stream) noexcept = 0;
+
+protected:
+    int32_t getTensorRTVersion() const noexcept override
+    {
+        return (static_cast<int32_t>(PluginVersion::kV2_DYNAMICEXT) << 24 | (NV_TENSORRT_VERSION & 0xFFFFFF));
+    }
+    virtual ~IPluginV2DynamicExt() noexcept {}
+
+private:
+    /* the static-shape methods of the bases are closed off, as in the reference */
+    void configurePlugin(Dims const*, int32_t, Dims const*, int32_t, DataType const*, DataType const*, bool const*,
+        bool const*, PluginFormat, int32_t) noexcept final
+    {
+    }
+    bool supportsFormat(DataType, PluginFormat) const noexcept final
+    {
+        return false;
+    }
+    Dims getOutputDimensions(int32_t, Dims const*, int32_t) noexcept final
+    {
+        return Dims{-1, {}};
+    }
+    size_t getWorkspaceSize(int32_t) const noexcept final
+    {
+        return 0;
+    }
+    int32_t enqueue(int32_t, void const* const*, void* const*, void*, hipStream_t) noexcept final
+    {
+        return 1;
+    }
+};
+
+class IPluginCreator : public IPluginCreatorInterface
+{
+public:
+    virtual AsciiChar const* getPluginName() const noexcept = 0;
+    virtual AsciiChar const* getPluginVersion() const noexcept = 0;
+    virtual PluginFieldCollection const* getFieldNames() noexcept = 0;
+    virtual IPluginV2* createPlugin(AsciiChar const* name, PluginFieldCollection const* fc) noexcept = 0;
+    virtual IPluginV2* deserializePlugin(AsciiChar const* name, void const* serialData, size_t serialLength) noexcept = 0;
+    virtual void setPluginNamespace(AsciiChar const* pluginNamespace) noexcept = 0;
+    virtual AsciiChar const* getPluginNamespace() const noexcept = 0;
+
+    IPluginCreator() = default;
+    ~IPluginCreator() override = default;
+
+protected:
+    IPluginCreator(IPluginCreator const&) = default;
+    IPluginCreator(IPluginCreator&&) = default;
+    IPluginCreator& operator=(IPluginCreator const&) & = default;
+    IPluginCreator& operator=(IPluginCreator&&) & = default;
+
+public:
+    InterfaceInfo getInterfaceInfo() const noexcept override
+    {
+        return InterfaceInfo{"PLUGIN CREATOR_V1", 1, 0};
+    }
 };
 } // namespace nvinfer1
 

@@ -93,6 +93,50 @@ TRTAMD_PLUGIN_API int32_t trtamd_plugin_enqueue(trtamd_plugin_t plugin, trtamd_t
  * valid until its next getFieldsToSerialize call or destruction. */
 TRTAMD_PLUGIN_API int32_t trtamd_plugin_fields_to_serialize(trtamd_plugin_t plugin, trtamd_plugin_field const** fields);
 
+/* ---- the deprecated IPluginV2DynamicExt / IPluginCreator versions ("Legacy" plugins of the reference:
+ *      emb 1-3, skip 1-4, qkv 1-3; plugin/bertQKVToContextPlugin/qkvToContextPluginLegacy.cpp:46-48 and
+ *      siblings).  One function per interface method, as above. ------------------------------------- */
+typedef void* trtamd_legacy_creator_t; /* nvinfer1::IPluginCreator* */
+typedef void* trtamd_legacy_plugin_t;  /* nvinfer1::IPluginV2DynamicExt* */
+
+/* registry lookup restricted to IPluginCreator ("PLUGIN CREATOR_V1") creators */
+TRTAMD_PLUGIN_API trtamd_legacy_creator_t trtamd_legacy_get_creator(char const* name, char const* version, char const* ns);
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_creator_field_names(trtamd_legacy_creator_t creator,
+    trtamd_plugin_field const** fields);
+/* IPluginCreator::createPlugin(name, fc) / deserializePlugin(name, data, length); NULL on failure */
+TRTAMD_PLUGIN_API trtamd_legacy_plugin_t trtamd_legacy_create(trtamd_legacy_creator_t creator, char const* layer_name,
+    trtamd_plugin_field const* fields, int32_t nb_fields);
+TRTAMD_PLUGIN_API trtamd_legacy_plugin_t trtamd_legacy_deserialize(trtamd_legacy_creator_t creator,
+    char const* layer_name, void const* data, size_t length);
+/* IPluginV2::destroy(), clone(), getPluginType(), getPluginVersion(), getNbOutputs(), getTensorRTVersion() */
+TRTAMD_PLUGIN_API void trtamd_legacy_destroy(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API trtamd_legacy_plugin_t trtamd_legacy_clone(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API char const* trtamd_legacy_type(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API char const* trtamd_legacy_version(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_nb_outputs(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_tensorrt_version(trtamd_legacy_plugin_t plugin);
+/* initialize() / terminate() */
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_initialize(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API void trtamd_legacy_terminate(trtamd_legacy_plugin_t plugin);
+/* getSerializationSize() / serialize(buffer) */
+TRTAMD_PLUGIN_API size_t trtamd_legacy_serialization_size(trtamd_legacy_plugin_t plugin);
+TRTAMD_PLUGIN_API void trtamd_legacy_serialize(trtamd_legacy_plugin_t plugin, void* buffer);
+/* getOutputDataType(index, inputTypes, nbInputs) */
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_output_type(
+    trtamd_legacy_plugin_t plugin, int32_t index, int32_t const* in_types, int32_t nb_inputs);
+/* getOutputDimensions(index, inputs, nbInputs, exprBuilder) with constant extents; returns 0 on success */
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_output_dims(trtamd_legacy_plugin_t plugin, int32_t index,
+    trtamd_tensor_desc const* in, int32_t nb_inputs, trtamd_tensor_desc* out);
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_supports_format(trtamd_legacy_plugin_t plugin, int32_t pos,
+    trtamd_tensor_desc const* in_out, int32_t nb_inputs, int32_t nb_outputs);
+TRTAMD_PLUGIN_API void trtamd_legacy_configure(trtamd_legacy_plugin_t plugin, trtamd_tensor_desc const* in,
+    int32_t nb_inputs, trtamd_tensor_desc const* out, int32_t nb_outputs);
+TRTAMD_PLUGIN_API size_t trtamd_legacy_workspace_size(trtamd_legacy_plugin_t plugin, trtamd_tensor_desc const* in,
+    int32_t nb_inputs, trtamd_tensor_desc const* out, int32_t nb_outputs);
+TRTAMD_PLUGIN_API int32_t trtamd_legacy_enqueue(trtamd_legacy_plugin_t plugin, trtamd_tensor_desc const* in,
+    int32_t nb_inputs, trtamd_tensor_desc const* out, int32_t nb_outputs, void const* const* inputs,
+    void* const* outputs, void* workspace, void* stream);
+
 /* Log capture: when enabled, an ILogger that remembers the last message of severity kERROR or
  * worse is installed (through initLibNvInferPlugins); trtamd_plugin_last_log returns that
  * message ("" if none) and clears it. */

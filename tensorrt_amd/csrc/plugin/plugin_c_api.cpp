@@ -213,7 +213,13 @@ CaptureLogger& captureLogger()
     return *logger;
 }
 
-IPluginCreatorV3One* creatorAt(int32_t index)
+bool isKind(IPluginCreatorInterface* c, char const* kind)
+{
+    InterfaceInfo const info = c->getInterfaceInfo();
+    return info.kind && std::string(info.kind) == kind;
+}
+
+IPluginCreatorInterface* creatorAt(int32_t index)
 {
     int32_t n = 0;
     IPluginCreatorInterface* const* list = getPluginRegistry()->getAllCreators(&n);
@@ -221,7 +227,12 @@ IPluginCreatorV3One* creatorAt(int32_t index)
     {
         return nullptr;
     }
-    return static_cast<IPluginCreatorV3One*>(list[index]);
+    return list[index];
+}
+
+IPluginV2DynamicExt* legacy(trtamd_legacy_plugin_t p)
+{
+    return static_cast<IPluginV2DynamicExt*>(p);
 }
 
 } // namespace
@@ -235,7 +246,7 @@ extern "C" {
 trtamd_creator_t trtamd_plugin_get_creator(char const* name, char const* version, char const* ns)
 {
     IPluginCreatorInterface* c = getPluginRegistry()->getCreator(name, version, ns ? ns : "");
-    return c ? static_cast<IPluginCreatorV3One*>(c) : nullptr;
+    return c && isKind(c, "PLUGIN CREATOR_V3ONE") ? static_cast<IPluginCreatorV3One*>(c) : nullptr;
 }
 
 int32_t trtamd_plugin_num_creators(void)
@@ -248,13 +259,23 @@ int32_t trtamd_plugin_num_creators(void)
 char const* trtamd_plugin_creator_name(int32_t index)
 {
     auto* c = creatorAt(index);
-    return c ? c->getPluginName() : nullptr;
+    if (!c)
+    {
+        return nullptr;
+    }
+    return isKind(c, "PLUGIN CREATOR_V1") ? static_cast<IPluginCreator*>(c)->getPluginName()
+                                           : static_cast<IPluginCreatorV3One*>(c)->getPluginName();
 }
 
 char const* trtamd_plugin_creator_version(int32_t index)
 {
     auto* c = creatorAt(index);
-    return c ? c->getPluginVersion() : nullptr;
+    if (!c)
+    {
+        return nullptr;
+    }
+    return isKind(c, "PLUGIN CREATOR_V1") ? static_cast<IPluginCreator*>(c)->getPluginVersion()
+                                           : static_cast<IPluginCreatorV3One*>(c)->getPluginVersion();
 }
 
 int32_t trtamd_plugin_creator_field_names(trtamd_creator_t creator, trtamd_plugin_field const** fields)
@@ -457,6 +478,210 @@ int32_t trtamd_plugin_fields_to_serialize(trtamd_plugin_t plugin, trtamd_plugin_
         *fields = reinterpret_cast<trtamd_plugin_field const*>(fc->fields);
     }
     return fc->nbFields;
+}
+
+// ---- IPluginCreator / IPluginV2DynamicExt -----------------------------------------------------------
+
+trtamd_legacy_creator_t trtamd_legacy_get_creator(char const* name, char const* version, char const* ns)
+{
+    IPluginCreatorInterface* c = getPluginRegistry()->getCreator(name, version, ns ? ns : "");
+    return c && isKind(c, "PLUGIN CREATOR_V1") ? static_cast<IPluginCreator*>(c) : nullptr;
+}
+
+int32_t trtamd_legacy_creator_field_names(trtamd_legacy_creator_t creator, trtamd_plugin_field const** fields)
+{
+    if (!creator)
+    {
+        return -1;
+    }
+    PluginFieldCollection const* fc = static_cast<IPluginCreator*>(creator)->getFieldNames();
+    if (!fc)
+    {
+        return -1;
+    }
+    if (fields)
+    {
+        *fields = reinterpret_cast<trtamd_plugin_field const*>(fc->fields);
+    }
+    return fc->nbFields;
+}
+
+trtamd_legacy_plugin_t trtamd_legacy_create(
+    trtamd_legacy_creator_t creator, char const* layer_name, trtamd_plugin_field const* fields, int32_t nb_fields)
+{
+    if (!creator)
+    {
+        return nullptr;
+    }
+    PluginFieldCollection fc{};
+    fc.nbFields = nb_fields;
+    fc.fields = reinterpret_cast<PluginField const*>(fields);
+    return static_cast<IPluginV2DynamicExt*>(static_cast<IPluginCreator*>(creator)->createPlugin(layer_name, &fc));
+}
+
+trtamd_legacy_plugin_t trtamd_legacy_deserialize(
+    trtamd_legacy_creator_t creator, char const* layer_name, void const* data, size_t length)
+{
+    if (!creator)
+    {
+        return nullptr;
+    }
+    return static_cast<IPluginV2DynamicExt*>(
+        static_cast<IPluginCreator*>(creator)->deserializePlugin(layer_name, data, length));
+}
+
+void trtamd_legacy_destroy(trtamd_legacy_plugin_t plugin)
+{
+    if (plugin)
+    {
+        legacy(plugin)->destroy();
+    }
+}
+
+trtamd_legacy_plugin_t trtamd_legacy_clone(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? legacy(plugin)->clone() : nullptr;
+}
+
+char const* trtamd_legacy_type(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? legacy(plugin)->getPluginType() : nullptr;
+}
+
+char const* trtamd_legacy_version(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? legacy(plugin)->getPluginVersion() : nullptr;
+}
+
+int32_t trtamd_legacy_nb_outputs(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? legacy(plugin)->getNbOutputs() : -1;
+}
+
+int32_t trtamd_legacy_tensorrt_version(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? static_cast<IPluginV2*>(legacy(plugin))->getTensorRTVersion() : -1;
+}
+
+int32_t trtamd_legacy_initialize(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? legacy(plugin)->initialize() : -1;
+}
+
+void trtamd_legacy_terminate(trtamd_legacy_plugin_t plugin)
+{
+    if (plugin)
+    {
+        legacy(plugin)->terminate();
+    }
+}
+
+size_t trtamd_legacy_serialization_size(trtamd_legacy_plugin_t plugin)
+{
+    return plugin ? legacy(plugin)->getSerializationSize() : 0;
+}
+
+void trtamd_legacy_serialize(trtamd_legacy_plugin_t plugin, void* buffer)
+{
+    if (plugin)
+    {
+        legacy(plugin)->serialize(buffer);
+    }
+}
+
+int32_t trtamd_legacy_output_type(trtamd_legacy_plugin_t plugin, int32_t index, int32_t const* in_types, int32_t nb_inputs)
+{
+    if (!plugin)
+    {
+        return -1;
+    }
+    std::vector<DataType> in(static_cast<size_t>(nb_inputs > 0 ? nb_inputs : 0));
+    for (int32_t i = 0; i < nb_inputs; ++i)
+    {
+        in[i] = static_cast<DataType>(in_types[i]);
+    }
+    return static_cast<int32_t>(legacy(plugin)->getOutputDataType(index, in.data(), nb_inputs));
+}
+
+int32_t trtamd_legacy_output_dims(trtamd_legacy_plugin_t plugin, int32_t index, trtamd_tensor_desc const* in,
+    int32_t nb_inputs, trtamd_tensor_desc* out)
+{
+    if (!plugin || nb_inputs < 0 || !out)
+    {
+        return -1;
+    }
+    FoldingBuilder builder;
+    std::vector<DimsExprs> ins(static_cast<size_t>(nb_inputs));
+    for (int32_t i = 0; i < nb_inputs; ++i)
+    {
+        ins[i].nbDims = in[i].nb_dims;
+        for (int32_t k = 0; k < in[i].nb_dims && k < TRTAMD_MAX_DIMS; ++k)
+        {
+            ins[i].d[k] = static_cast<IExprBuilder&>(builder).constant(in[i].dims[k]);
+        }
+    }
+    DimsExprs const d = legacy(plugin)->getOutputDimensions(index, ins.data(), nb_inputs, builder);
+    if (d.nbDims < 0)
+    {
+        return -1;
+    }
+    out->nb_dims = d.nbDims;
+    for (int32_t k = 0; k < d.nbDims && k < TRTAMD_MAX_DIMS; ++k)
+    {
+        if (!d.d[k])
+        {
+            return -1;
+        }
+        out->dims[k] = d.d[k]->getConstantValue();
+    }
+    return 0;
+}
+
+int32_t trtamd_legacy_supports_format(
+    trtamd_legacy_plugin_t plugin, int32_t pos, trtamd_tensor_desc const* in_out, int32_t nb_inputs, int32_t nb_outputs)
+{
+    if (!plugin)
+    {
+        return 0;
+    }
+    auto v = toDescs(in_out, nb_inputs + nb_outputs);
+    return legacy(plugin)->supportsFormatCombination(pos, v.data(), nb_inputs, nb_outputs) ? 1 : 0;
+}
+
+void trtamd_legacy_configure(trtamd_legacy_plugin_t plugin, trtamd_tensor_desc const* in, int32_t nb_inputs,
+    trtamd_tensor_desc const* out, int32_t nb_outputs)
+{
+    if (plugin)
+    {
+        auto i = toDynDescs(in, nb_inputs);
+        auto o = toDynDescs(out, nb_outputs);
+        legacy(plugin)->configurePlugin(i.data(), nb_inputs, o.data(), nb_outputs);
+    }
+}
+
+size_t trtamd_legacy_workspace_size(trtamd_legacy_plugin_t plugin, trtamd_tensor_desc const* in, int32_t nb_inputs,
+    trtamd_tensor_desc const* out, int32_t nb_outputs)
+{
+    if (!plugin)
+    {
+        return 0;
+    }
+    auto i = toDescs(in, nb_inputs);
+    auto o = toDescs(out, nb_outputs);
+    return legacy(plugin)->getWorkspaceSize(i.data(), nb_inputs, o.data(), nb_outputs);
+}
+
+int32_t trtamd_legacy_enqueue(trtamd_legacy_plugin_t plugin, trtamd_tensor_desc const* in, int32_t nb_inputs,
+    trtamd_tensor_desc const* out, int32_t nb_outputs, void const* const* inputs, void* const* outputs, void* workspace,
+    void* stream)
+{
+    if (!plugin)
+    {
+        return -1;
+    }
+    auto i = toDescs(in, nb_inputs);
+    auto o = toDescs(out, nb_outputs);
+    return legacy(plugin)->enqueue(i.data(), o.data(), inputs, outputs, workspace, static_cast<hipStream_t>(stream));
 }
 
 void trtamd_plugin_capture_log(int32_t enable)

@@ -206,20 +206,33 @@ private:
 
     bool addLocked(IPluginCreatorInterface& creator, std::string const& ns, void* library)
     {
-        // only IPluginCreatorV3One creators carry a name and a version this registry can key on
+        // IPluginCreatorV3One and the deprecated IPluginCreator carry a name and a version to key on
         InterfaceInfo const info = creator.getInterfaceInfo();
-        if (!info.kind || std::string(info.kind) != "PLUGIN CREATOR_V3ONE")
+        std::string const kind = info.kind ? info.kind : "";
+        char const* name = nullptr;
+        char const* version = nullptr;
+        if (kind == "PLUGIN CREATOR_V3ONE")
+        {
+            auto& c = static_cast<IPluginCreatorV3One&>(creator);
+            name = c.getPluginName();
+            version = c.getPluginVersion();
+        }
+        else if (kind == "PLUGIN CREATOR_V1")
+        {
+            auto& c = static_cast<IPluginCreator&>(creator);
+            name = c.getPluginName();
+            version = c.getPluginVersion();
+        }
+        if (!name || !version)
         {
             logMessage(ILogger::Severity::kERROR, "registerCreator: unsupported creator interface");
             return false;
         }
-        auto& c = static_cast<IPluginCreatorV3One&>(creator);
-        Key key{ns, c.getPluginName(), c.getPluginVersion()};
+        Key key{ns, name, version};
         if (mCreators.count(key))
         {
             logMessage(ILogger::Severity::kVERBOSE,
-                std::string("Plugin creator already registered - ") + c.getPluginName() + " version "
-                    + c.getPluginVersion());
+                std::string("Plugin creator already registered - ") + name + " version " + version);
             return false;
         }
         mCreators.emplace(std::move(key), Entry{&creator, library});

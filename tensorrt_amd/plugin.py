@@ -156,6 +156,26 @@ def _library():
         "trtamd_plugin_on_shape_change": (i32, [vp, pd, i32, pd, i32]),
         "trtamd_plugin_enqueue": (i32, [vp, pd, i32, pd, i32, C.POINTER(vp), C.POINTER(vp), vp, vp]),
         "trtamd_plugin_fields_to_serialize": (i32, [vp, C.POINTER(pf)]),
+        "trtamd_legacy_get_creator": (vp, [C.c_char_p, C.c_char_p, C.c_char_p]),
+        "trtamd_legacy_creator_field_names": (i32, [vp, C.POINTER(pf)]),
+        "trtamd_legacy_create": (vp, [vp, C.c_char_p, pf, i32]),
+        "trtamd_legacy_deserialize": (vp, [vp, C.c_char_p, C.c_void_p, C.c_size_t]),
+        "trtamd_legacy_destroy": (None, [vp]),
+        "trtamd_legacy_clone": (vp, [vp]),
+        "trtamd_legacy_type": (C.c_char_p, [vp]),
+        "trtamd_legacy_version": (C.c_char_p, [vp]),
+        "trtamd_legacy_nb_outputs": (i32, [vp]),
+        "trtamd_legacy_tensorrt_version": (i32, [vp]),
+        "trtamd_legacy_initialize": (i32, [vp]),
+        "trtamd_legacy_terminate": (None, [vp]),
+        "trtamd_legacy_serialization_size": (C.c_size_t, [vp]),
+        "trtamd_legacy_serialize": (None, [vp, C.c_void_p]),
+        "trtamd_legacy_output_type": (i32, [vp, i32, C.POINTER(i32), i32]),
+        "trtamd_legacy_output_dims": (i32, [vp, i32, pd, i32, pd]),
+        "trtamd_legacy_supports_format": (i32, [vp, i32, pd, i32, i32]),
+        "trtamd_legacy_configure": (None, [vp, pd, i32, pd, i32]),
+        "trtamd_legacy_workspace_size": (C.c_size_t, [vp, pd, i32, pd, i32]),
+        "trtamd_legacy_enqueue": (i32, [vp, pd, i32, pd, i32, C.POINTER(vp), C.POINTER(vp), vp, vp]),
         "trtamd_plugin_capture_log": (None, [i32]),
         "trtamd_plugin_last_log": (C.c_char_p, []),
     }
@@ -285,6 +305,124 @@ class Plugin:
         return _fields_from_c(ptr, n)
 
 
+class LegacyPlugin:
+    """An IPluginV2DynamicExt instance (one of the reference's "Legacy" plugin versions)."""
+
+    def __init__(self, handle: int):
+        self._h = handle
+        self._lib = _library()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.trtamd_legacy_destroy(self._h)
+            self._h = None
+
+    # IPluginV2
+    @property
+    def plugin_type(self) -> str:
+        return self._lib.trtamd_legacy_type(self._h).decode()
+
+    @property
+    def plugin_version(self) -> str:
+        return self._lib.trtamd_legacy_version(self._h).decode()
+
+    @property
+    def num_outputs(self) -> int:
+        return self._lib.trtamd_legacy_nb_outputs(self._h)
+
+    @property
+    def tensorrt_version(self) -> int:
+        return self._lib.trtamd_legacy_tensorrt_version(self._h)
+
+    def initialize(self) -> int:
+        return self._lib.trtamd_legacy_initialize(self._h)
+
+    def terminate(self) -> None:
+        self._lib.trtamd_legacy_terminate(self._h)
+
+    def get_serialization_size(self) -> int:
+        return int(self._lib.trtamd_legacy_serialization_size(self._h))
+
+    def serialize(self) -> bytes:
+        n = self.get_serialization_size()
+        buf = C.create_string_buffer(max(n, 1))
+        self._lib.trtamd_legacy_serialize(self._h, buf)
+        return buf.raw[:n]
+
+    def clone(self) -> "LegacyPlugin | None":
+        h = self._lib.trtamd_legacy_clone(self._h)
+        return LegacyPlugin(h) if h else None
+
+    # IPluginV2Ext
+    def get_output_data_type(self, index: int, input_types: Sequence[DataType]) -> DataType:
+        inp = (C.c_int32 * max(len(input_types), 1))(*[int(t) for t in input_types])
+        return DataType(self._lib.trtamd_legacy_output_type(self._h, index, inp, len(input_types)))
+
+    # IPluginV2DynamicExt
+    def get_output_dimensions(self, index: int, inputs: Sequence[TensorDesc]):
+        cin, n = _descs(inputs)
+        cout = (_CDesc * 1)()
+        if self._lib.trtamd_legacy_output_dims(self._h, index, cin, n, cout) != 0:
+            return None
+        return [int(cout[0].dims[k]) for k in range(cout[0].nb_dims)]
+
+    def supports_format_combination(self, pos: int, in_out: Sequence[TensorDesc], num_inputs: int) -> bool:
+        c, n = _descs(in_out)
+        return bool(self._lib.trtamd_legacy_supports_format(self._h, pos, c, num_inputs, n - num_inputs))
+
+    def configure_plugin(self, inputs: Sequence[TensorDesc], outputs: Sequence[TensorDesc]) -> None:
+        ci, ni = _descs(inputs)
+        co, no = _descs(outputs)
+        self._lib.trtamd_legacy_configure(self._h, ci, ni, co, no)
+
+    def get_workspace_size(self, inputs: Sequence[TensorDesc], outputs: Sequence[TensorDesc]) -> int:
+        ci, ni = _descs(inputs)
+        co, no = _descs(outputs)
+        return int(self._lib.trtamd_legacy_workspace_size(self._h, ci, ni, co, no))
+
+    def enqueue(self, input_desc: Sequence[TensorDesc], output_desc: Sequence[TensorDesc], inputs: Sequence[int],
+                outputs: Sequence[int], workspace: int = 0, stream: int = 0) -> int:
+        ci, ni = _descs(input_desc)
+        co, no = _descs(output_desc)
+        pin = (C.c_void_p * max(len(inputs), 1))(*[C.c_void_p(int(p)) for p in inputs])
+        pout = (C.c_void_p * max(len(outputs), 1))(*[C.c_void_p(int(p)) for p in outputs])
+        return self._lib.trtamd_legacy_enqueue(self._h, ci, ni, co, no, pin, pout, C.c_void_p(int(workspace)),
+                                               C.c_void_p(int(stream)))
+
+
+class LegacyPluginCreator:
+    """An IPluginCreator (owned by the registry)."""
+
+    def __init__(self, handle: int):
+        self._h = handle
+        self._lib = _library()
+
+    @property
+    def field_names(self) -> list[PluginField]:
+        ptr = C.POINTER(_CField)()
+        n = self._lib.trtamd_legacy_creator_field_names(self._h, C.byref(ptr))
+        return _fields_from_c(ptr, max(n, 0))
+
+    def create_plugin(self, name: str, fc) -> LegacyPlugin | None:
+        fields = list(fc)
+        arr = (_CField * max(len(fields), 1))()
+        keep = []
+        for i, f in enumerate(fields):
+            nm = f.name.encode()
+            keep.append(nm)
+            arr[i].name = nm
+            arr[i].data = f.data.ctypes.data if f.data is not None else None
+            arr[i].type = int(f.type)
+            arr[i].length = f.length
+        h = self._lib.trtamd_legacy_create(self._h, name.encode(), arr, len(fields))
+        return LegacyPlugin(h) if h else None
+
+    def deserialize_plugin(self, name: str, data: bytes) -> LegacyPlugin | None:
+        buf = C.create_string_buffer(data, len(data))
+        h = self._lib.trtamd_legacy_deserialize(self._h, name.encode(), buf, len(data))
+        return LegacyPlugin(h) if h else None
+
+
 @dataclass
 class PluginFieldCollection:
     fields: list[PluginField] = field(default_factory=list)
@@ -331,6 +469,11 @@ class PluginRegistry:
     def get_creator(self, name: str, version: str, plugin_namespace: str = "") -> PluginCreator | None:
         h = self._lib.trtamd_plugin_get_creator(name.encode(), version.encode(), plugin_namespace.encode())
         return PluginCreator(h) if h else None
+
+    def get_legacy_creator(self, name: str, version: str, plugin_namespace: str = "") -> LegacyPluginCreator | None:
+        """The IPluginCreator registered under (name, version), if that version is a legacy one."""
+        h = self._lib.trtamd_legacy_get_creator(name.encode(), version.encode(), plugin_namespace.encode())
+        return LegacyPluginCreator(h) if h else None
 
     @property
     def all_creators(self) -> list[tuple[str, str]]:

@@ -55,9 +55,11 @@ def roundtrip(creator, plugin, name="rt"):
 # ---- registry --------------------------------------------------------------------------------------
 
 def test_all_creators_registered(reg):
-    want = {(SKIPLN, v) for v in "5678"} | {(EMBLN, v) for v in "456"} | {(QKV, v) for v in "456"}
+    want = {(SKIPLN, v) for v in "12345678"} | {(EMBLN, v) for v in "123456"} | {(QKV, v) for v in "123456"}
     assert set(reg.all_creators) == want
-    assert reg.get_creator(SKIPLN, "1") is None          # the IPluginV2 generations are not provided
+    # versions 1..(3|4) are IPluginCreator objects, the later ones IPluginCreatorV3One: each lookup sees its own kind
+    assert reg.get_creator(SKIPLN, "1") is None and reg.get_legacy_creator(SKIPLN, "1") is not None
+    assert reg.get_legacy_creator(SKIPLN, "5") is None
     assert reg.get_creator(SKIPLN, "5", "other_ns") is None
     assert reg.get_creator("NoSuchPlugin", "1") is None
 
@@ -440,3 +442,106 @@ def test_enqueue_without_a_gpu_fails_cleanly(reg):
     d = TensorDesc([4, 1, 768, 1, 1], DataType.HALF)
     assert p.enqueue([d, d], [d], [0, 0], [0]) != 0
     assert last_log() != ""
+
+
+# ---- the IPluginV2DynamicExt ("Legacy") versions ------------------------------------------------------
+
+LEGACY = [(SKIPLN, "1", "5"), (SKIPLN, "2", "6"), (SKIPLN, "3", "7"), (SKIPLN, "4", "8"),
+          (EMBLN, "1", "6"), (EMBLN, "2", "4"), (EMBLN, "3", "5"),
+          (QKV, "1", "4"), (QKV, "2", "5"), (QKV, "3", "6")]
+
+
+def legacy_fields(name, version):
+    r = np.random.default_rng(5)
+    if name == SKIPLN:
+        ld = 768
+        fs = [PluginField("beta", r.standard_normal(ld).astype(np.float32), F32),
+              PluginField("gamma", r.standard_normal(ld).astype(np.float32), F32)]
+        if version in "12":
+            fs += [i32("type_id", 1), PluginField("bias", r.standard_normal(ld).astype(np.float32), F32)]
+        if version == "1":
+            fs.append(i32("ld", ld))
+        return fs
+    if name == EMBLN:
+        ld = 128
+        fs = [PluginField("bert_embeddings_layernorm_beta", r.standard_normal(ld).astype(np.float32), F32),
+              PluginField("bert_embeddings_layernorm_gamma", r.standard_normal(ld).astype(np.float32), F32),
+              PluginField("bert_embeddings_word_embeddings", r.standard_normal((50, ld)).astype(np.float32), F32),
+              PluginField("bert_embeddings_token_type_embeddings", r.standard_normal((2, ld)).astype(np.float32), F32),
+              PluginField("bert_embeddings_position_embeddings", r.standard_normal((64, ld)).astype(np.float32), F32),
+              i32("output_fp16", 1)]
+        if version == "1":
+            fs += [i32("full_mask", 0), i32("mha_type_id", 1)]
+        return fs
+    if version == "3":
+        return [i32("hidden_size", 1024), i32("num_heads", 16), f32("dq_probs", 1 / 127)]
+    fs = [i32("type_id", 1), i32("hidden_size", 768), i32("num_heads", 12), i32("has_mask", 1)]
+    if version == "2":
+        fs.append(i32("var_seqlen", 1))
+    return fs
+
+
+@pytest.mark.parametrize("name,legacy,current", LEGACY)
+def test_legacy_versions_wrap_the_current_plugins(reg, name, legacy, current):
+    """Versions and creator fields of the reference's *Legacy.cpp files; same behaviour as the V3 version."""
+    lc = reg.get_legacy_creator(name, legacy)
+    cc = reg.get_creator(name, current)
+    assert lc is not None and cc is not None
+    assert sorted(f.name for f in lc.field_names) == sorted(f.name for f in cc.field_names)
+    fs = legacy_fields(name, legacy)
+    p = lc.create_plugin("layer", fs)
+    assert p is not None, last_log()
+    ref = cc.create_plugin("layer", fs, TensorRTPhase.BUILD)
+    assert p.plugin_type == name and p.plugin_version == legacy
+    assert p.num_outputs == ref.num_outputs
+    # IPluginV2DynamicExt::getTensorRTVersion: PluginVersion::kV2_DYNAMICEXT in the top byte, TensorRT 11.1.0 below
+    assert p.tensorrt_version == (3 << 24) | 110100
+    assert p.initialize() == 0
+    p.terminate()
+    if name == QKV and legacy != "3":
+        # the attention plugins serialise the runner chosen in configurePlugin (S, B), as the reference's do
+        if legacy == "1":
+            ins = [TensorDesc([128, 2, 3 * 768, 1, 1], DataType.HALF), TensorDesc([2, 512], DataType.INT32)]
+            outs = [TensorDesc([128, 2, 768, 1, 1], DataType.HALF)]
+        else:
+            ins = [TensorDesc([300, 3 * 768, 1, 1], DataType.HALF), TensorDesc([1], DataType.INT32),
+                   TensorDesc([5], DataType.INT32), TensorDesc([128], DataType.INT32)]
+            outs = [TensorDesc([300, 768, 1, 1], DataType.HALF)]
+        p.configure_plugin(ins, outs)
+
+    # serialize -> deserializePlugin -> serialize reproduces the bytes; a clone serialises to the same bytes
+    blob = p.serialize()
+    assert len(blob) == p.get_serialization_size() > 0
+    q = lc.deserialize_plugin("layer", blob)
+    assert q is not None, last_log()
+    assert q.plugin_version == legacy and q.serialize() == blob
+    assert p.clone().serialize() == blob
+    # a damaged stream is refused with a message, not a crash
+    assert lc.deserialize_plugin("layer", blob[: len(blob) // 2]) is None
+    assert "truncated" in last_log()
+    assert lc.deserialize_plugin("layer", b"\0" * 64) is None
+    last_log()
+
+
+def test_legacy_skipln_shapes_types_formats(reg):
+    lc = reg.get_legacy_creator(SKIPLN, "1")
+    p = lc.create_plugin("sln", legacy_fields(SKIPLN, "1"))
+    shape = [128, 4, 768, 1, 1]
+    half = TensorDesc(shape, DataType.HALF)
+    assert p.get_output_dimensions(0, [half, half]) == shape
+    assert p.get_output_dimensions(1, [half, half]) is None
+    assert p.get_output_data_type(0, [DataType.HALF, DataType.HALF]) == DataType.HALF
+    assert p.supports_format_combination(0, [half, half, half], 2)
+    assert p.supports_format_combination(2, [half, half, half], 2)
+    assert not p.supports_format_combination(1, [half, TensorDesc(shape, DataType.FLOAT), half], 2)
+    assert p.get_workspace_size([half, half], [half]) == 0
+
+
+def test_legacy_enqueue_without_a_gpu_fails_cleanly(reg):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lc = reg.get_legacy_creator(SKIPLN, "3")
+    p = lc.create_plugin("sln", legacy_fields(SKIPLN, "3"))
+    d = TensorDesc([1, 768, 64, 1], DataType.INT8, TensorFormat.CHW32, 0.1)
+    assert p.enqueue([d, d], [d], [0, 0], [0]) != 0
