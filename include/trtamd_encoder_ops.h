@@ -55,6 +55,25 @@ typedef struct trtamd_int8_linear_params
  * (closed source; engine-side placement described in plugin/bertQKVToContextPlugin/README.md:25-30). */
 TRTAMD_API int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_params const* params);
 
+/* FP16 linear layer for the FP16 encoder: out[t][n] = binary16(f(fmaf(acc, alpha[n], beta[n]))), acc = sum_k
+ * a[t][k] * w[n][k] accumulated in binary32 on the FP16 matrix cores, f = identity (TRTAMD_LINEAR_AFFINE) or erf-GELU
+ * (TRTAMD_LINEAR_GELU).  alpha = 1 and beta = bias give the usual fully-connected layer.  All tensors linear:
+ * a [T][K], w [N][K], out [T][N]; K % 32 == 0, N % 32 == 0.  The open counterpart in the reference is the deprecated
+ * cuBLASLt GEMM plugin CustomFCPluginDynamic (plugin/fcPlugin/README.md:20-45, FP16 without bias or activation);
+ * bias and GELU are what TensorRT's core fuses onto it. */
+typedef struct trtamd_fp16_linear_params
+{
+    trtamd_half_t const* a;
+    trtamd_half_t const* w;
+    float const* alpha; /* [N] */
+    float const* beta;  /* [N] */
+    trtamd_half_t* out;
+    int32_t T, K, N;
+    int32_t epilogue;   /* TRTAMD_LINEAR_AFFINE or TRTAMD_LINEAR_GELU */
+} trtamd_fp16_linear_params;
+
+TRTAMD_API int trtamd_fp16_linear(trtamd_stream_t stream, trtamd_fp16_linear_params const* params);
+
 /* ------------------------------------------------------------------------------------------
  * Reformats either side of the interleaved plugins.  TensorRT inserts these itself when a plugin asks
  * for TensorFormat::kCHW32 (include/NvInferRuntime.h:1471; the INT8 interleaved plugins do:

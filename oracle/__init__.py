@@ -352,3 +352,16 @@ def dequantize_deinterleave_f16(q, scale):
     out = np.zeros((T, nslab * 32), np.float16)
     lib().orc_dequantize_deinterleave_f16(_p(q), C.c_float(scale), _p(out), C.c_int64(T), C.c_int(nslab * 32))
     return out
+
+
+def fp16_linear(a, w, alpha, beta, gelu=False):
+    """a: float16 [T,K]; w: float16 [N,K]; alpha, beta: float32 [N].  Returns float16 [T,N]."""
+    a, w = _c(a, np.float16), _c(w, np.float16)
+    T, K = a.shape
+    N = w.shape[0]
+    out = np.zeros((T, N), np.float16)
+    rc = lib().orc_fp16_linear(C.c_int64(T), C.c_int(K), C.c_int(N), _p(a), _p(w), _p(_c(alpha, np.float32)),
+                               _p(_c(beta, np.float32)), C.c_int(int(gelu)), _p(out))
+    if rc != 0:
+        raise ValueError("orc_fp16_linear rejected its arguments")
+    return out

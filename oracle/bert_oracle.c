@@ -1187,3 +1187,49 @@ ORC_API void orc_dequantize_deinterleave_f16(int8_t const* q, float scale, uint1
         }
     }
 }
+
+/* FP16 linear layer (include/trtamd_encoder_ops.h, trtamd_fp16_linear): the arithmetic of a cuBLASLt FP16 GEMM
+ * with binary32 accumulation as CustomFCPluginDynamic configures it (plugin/fcPlugin/fcPlugin.cpp, compute type
+ * CUBLAS_COMPUTE_32F for DataType::kHALF), plus the bias / GELU TensorRT fuses after it:
+ *   acc = sum_k a[t][k] * w[n][k] in binary32 (products of binary16 values are exact in binary32; the order of
+ *   the additions is k = 0, 1, ... here and a tree on the GPU, hence the floating-point tolerance of the tests)
+ *   y = fmaf(acc, alpha[n], beta[n]);  epilogue 1: y = 0.5 y (1 + erf(y / sqrt 2)) in binary64;  out = binary16(y). */
+ORC_API int orc_fp16_linear(int64_t T, int K, int N, uint16_t const* a, uint16_t const* w, float const* alpha,
+    float const* beta, int epilogue, uint16_t* out)
+{
+    if (K <= 0 || N <= 0 || epilogue < 0 || epilogue > 1)
+    {
+        return 1;
+    }
+    float* wf = (float*) malloc((size_t) N * K * sizeof(float));
+    for (int64_t i = 0; i < (int64_t) N * K; ++i)
+    {
+        wf[i] = h2f(w[i]);
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t)
+    {
+        float* row = (float*) malloc((size_t) K * sizeof(float));
+        for (int k = 0; k < K; ++k)
+        {
+            row[k] = h2f(a[t * K + k]);
+        }
+        for (int n = 0; n < N; ++n)
+        {
+            float acc = 0.f;
+            for (int k = 0; k < K; ++k)
+            {
+                acc += row[k] * wf[(int64_t) n * K + k];
+            }
+            double y = (double) fmaf(acc, alpha[n], beta[n]);
+            if (epilogue == 1)
+            {
+                y = 0.5 * y * (1.0 + erf(y * 0.70710678118654752440));
+            }
+            out[t * N + n] = d2h(y);
+        }
+        free(row);
+    }
+    free(wf);
+    return 0;
+}

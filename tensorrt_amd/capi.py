@@ -41,6 +41,14 @@ class Int8LinearParams(C.Structure):
     ]
 
 
+class Fp16LinearParams(C.Structure):
+    """struct trtamd_fp16_linear_params (include/trtamd_encoder_ops.h)."""
+    _fields_ = [
+        ("a", c_p), ("w", c_p), ("alpha", c_p), ("beta", c_p), ("out", c_p),
+        ("T", i32), ("K", i32), ("N", i32), ("epilogue", i32),
+    ]
+
+
 LINEAR_AFFINE, LINEAR_GELU, LINEAR_RAW_INT32, LINEAR_AFFINE_FP16 = 0, 1, 2, 3
 
 _SIGS = {
@@ -76,6 +84,7 @@ _SIGS = {
     "trtamd_fused_mha_is_valid": (C.c_int, [i32, i32, i32]),
     "trtamd_zero_padding_2d": (C.c_int, [c_p, i32, c_p, i32, i32, c_p]),
     "trtamd_int8_linear": (C.c_int, [c_p, C.POINTER(Int8LinearParams)]),
+    "trtamd_fp16_linear": (C.c_int, [c_p, C.POINTER(Fp16LinearParams)]),
     "trtamd_int8_linear_to_interleaved": (C.c_int, [c_p, i32, i32, c_p, c_p]),
     "trtamd_int8_interleaved_to_linear": (C.c_int, [c_p, i32, i32, c_p, c_p]),
     "trtamd_quantize_fp16_to_interleaved": (C.c_int, [c_p, i32, i32, c_p, f32, c_p]),
@@ -84,7 +93,7 @@ _SIGS = {
 
 # Entry points declared in include/trtamd_bert_kernels.h (the debug hook is extra).
 # Entry points declared in include/trtamd_encoder_ops.h.
-ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear", "trtamd_int8_linear_to_interleaved", "trtamd_int8_interleaved_to_linear",
+ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear", "trtamd_fp16_linear", "trtamd_int8_linear_to_interleaved", "trtamd_int8_interleaved_to_linear",
                        "trtamd_quantize_fp16_to_interleaved", "trtamd_dequantize_interleaved_to_fp16"]
 HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug" and k not in ENCODER_OPS_SYMBOLS]
 

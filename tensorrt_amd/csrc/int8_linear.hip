@@ -40,8 +40,30 @@ enum Epilogue
     kAFFINE = TRTAMD_LINEAR_AFFINE,
     kGELU = TRTAMD_LINEAR_GELU,
     kRAW = TRTAMD_LINEAR_RAW_INT32,
-    kHALF = TRTAMD_LINEAR_AFFINE_FP16
+    kHALF = TRTAMD_LINEAR_AFFINE_FP16,
+    // FP16 operands (trtamd_fp16_linear): the same kernels with v_mfma_f32_32x32x16_f16 and binary32 accumulators
+    kF16_AFFINE = 4,
+    kF16_GELU = 5
 };
+
+// INT8 operands accumulate in INT32, FP16 operands in binary32.  Either way a lane feeds 16 bytes of a row per
+// operand and MFMA step (16 INT8 or 8 FP16 values of k), a fragment is 32 rows x 32 bytes, and the result has the
+// same 32 x 32 accumulator layout, so the tiling, the LDS layout and the load schedule are shared.
+template <int EPI>
+using AccT = std::conditional_t<(EPI >= kF16_AFFINE), f32x16, i32x16>;
+
+template <int EPI>
+__device__ __forceinline__ AccT<EPI> mma(i32x4 const a, i32x4 const b, AccT<EPI> const c)
+{
+    if constexpr (EPI >= kF16_AFFINE)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(bits_as<f16x8>(a), bits_as<f16x8>(b), c, 0, 0, 0);
+    }
+    else
+    {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    }
+}
 
 struct LinearArgs
 {
@@ -50,7 +72,7 @@ struct LinearArgs
     float const* alpha;
     float const* beta;
     void* out;
-    int T, K, N;
+    int T, K, N; // K: bytes of k per row (elements for INT8, twice the elements for FP16)
     float qOut;
     int mainTiles; // workgroups that own a 256 x 256 tile
     int tokMain;   // rows of 256 tokens they cover
@@ -107,7 +129,7 @@ __device__ inline int frag_offset(int row, int half)
 // that share a token trade two packed dwords (v_permlane32_swap), after which lane l holds the 16
 // consecutive channels 16*(l/32)..+15 and stores them with one 16-byte write.
 template <int WM, int WN, int MT, int NT, bool IL_OUT, int EPI>
-__device__ __forceinline__ void store_tile(LinearArgs const& p, i32x16 const (&acc)[MT][NT], int const n0, int const t0,
+__device__ __forceinline__ void store_tile(LinearArgs const& p, AccT<EPI> const (&acc)[MT][NT], int const n0, int const t0,
     float const* sAlpha, float const* sBeta)
 {
     int const lane = threadIdx.x & 63;
@@ -151,6 +173,25 @@ __device__ __forceinline__ void store_tile(LinearArgs const& p, i32x16 const (&a
                         *reinterpret_cast<i32x4*>(
                             static_cast<int32_t*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
                             = v;
+                    }
+                }
+            }
+            else if constexpr (EPI >= kF16_AFFINE)
+            {
+                if (live)
+                {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        f16x4 h;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            float const y = fmaf(acc[i][j][4 * g + e], al[g][e], be[g][e]);
+                            h[e] = (f16) (EPI == kF16_GELU ? gelu_erf(y) : y);
+                        }
+                        *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
+                            = h;
                     }
                 }
             }
@@ -301,7 +342,7 @@ __device__ __forceinline__ void linear_tile(
         }
     };
 
-    i32x16 acc[MT][NT];
+    AccT<EPI> acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
     {
@@ -338,7 +379,7 @@ __device__ __forceinline__ void linear_tile(
 #pragma unroll
                 for (int j = 0; j < NT; ++j)
                 {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = mma<EPI>(fa[i], fb[j], acc[i][j]);
                 }
             }
         }
@@ -472,7 +513,7 @@ __device__ __forceinline__ void linear_tile_run(
         }
     };
 
-    i32x16 acc[MT][NT];
+    AccT<EPI> acc[MT][NT];
     int const readOff = frag_offset(lane & 31, lane >> 5);
     auto multiply = [&](int buf) {
         uint8_t const* base = lds + buf * STAGE + readOff;
@@ -496,7 +537,7 @@ __device__ __forceinline__ void linear_tile_run(
 #pragma unroll
                 for (int j = 0; j < NT; ++j)
                 {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = mma<EPI>(fa[i], fb[j], acc[i][j]);
                 }
             }
         }
@@ -681,12 +722,9 @@ int launch_shape(hipStream_t stream, LinearArgs a)
     int const cus = num_cus();
     a.tokMain = (int) ((bigTiles / cus) * cus / nbmBig);
     a.mainTiles = a.tokMain * nbmBig;
-    static int const maxPanel = [] {
-        char const* e = getenv("TRTAMD_LINEAR_PANEL");
-        return e ? atoi(e) : 8;
-    }();
+    constexpr int kMaxPanel = 8; // 8 x 256 channels x K = 1024 of weights is half of an XCD's 4 MB L2
     a.panel = 1;
-    for (int w = 1; w <= maxPanel && w <= nbmBig; ++w)
+    for (int w = 1; w <= kMaxPanel && w <= nbmBig; ++w)
     {
         if (nbmBig % w == 0)
         {
@@ -779,4 +817,40 @@ extern "C" int trtamd_int8_linear(trtamd_stream_t stream, trtamd_int8_linear_par
     }
     return p->a_interleaved ? launch_out<false, true>(st, a, p->epilogue, ilOut)
                             : launch_out<false, false>(st, a, p->epilogue, ilOut);
+}
+
+extern "C" int trtamd_fp16_linear(trtamd_stream_t stream, trtamd_fp16_linear_params const* p)
+{
+    using namespace trtamd;
+    if (p == nullptr || p->a == nullptr || p->w == nullptr || p->out == nullptr || p->alpha == nullptr
+        || p->beta == nullptr)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "fp16_linear: null pointer");
+    }
+    if (p->T < 0 || p->K <= 0 || p->N <= 0 || p->K % 32 != 0 || p->N % 32 != 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "fp16_linear: T=%d K=%d N=%d (K and N must be multiples of 32)", p->T,
+            p->K, p->N);
+    }
+    if (p->epilogue != TRTAMD_LINEAR_AFFINE && p->epilogue != TRTAMD_LINEAR_GELU)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "fp16_linear: unknown epilogue %d", p->epilogue);
+    }
+    if ((int64_t) p->T * p->K >= (int64_t) 1 << 30 || (int64_t) p->N * p->K >= (int64_t) 1 << 30)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "fp16_linear: operand of 2 GiB or more");
+    }
+    if (!aligned16(p->a) || !aligned16(p->w) || !aligned16(p->out) || !aligned16(p->alpha) || !aligned16(p->beta))
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "fp16_linear: pointers must be 16-byte aligned");
+    }
+    if (p->T == 0)
+    {
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    LinearArgs a{reinterpret_cast<int8_t const*>(p->a), reinterpret_cast<int8_t const*>(p->w), p->alpha, p->beta, p->out,
+        p->T, 2 * p->K, p->N, 1.f, 0, 0, 1, 0};
+    hipStream_t const st = as_stream(stream);
+    return p->epilogue == TRTAMD_LINEAR_GELU ? launch_shape<false, false, false, kF16_GELU>(st, a)
+                                             : launch_shape<false, false, false, kF16_AFFINE>(st, a);
 }

@@ -302,9 +302,8 @@ class Int8BertEncoder:
         # a normalised row has |z| <= sqrt(E); start wide, measure, tighten
         gamma, beta = L[ln + "_gamma"].astype(np.float32), L[ln + "_beta"].astype(np.float32)
         wide = float(np.float32((8.0 * np.abs(gamma).max() + np.abs(beta).max()) / 127.0))
-        tmp = self.torch.empty_like(dst) if dst.data_ptr() == skip.data_ptr() else dst
-        self._skipln(L[ln], src, s_src, skip, s_skip, tmp, wide)
-        s = float(np.float32(wide * max(self._amax_int8(tmp), 1) * margin / 127.0))
+        self._skipln(L[ln], src, s_src, skip, s_skip, dst, wide)
+        s = float(np.float32(wide * max(self._amax_int8(dst), 1) * margin / 127.0))
         self._skipln(L[ln], src, s_src, skip, s_skip, dst, s)
         return s
 

@@ -196,6 +196,21 @@ def main():
         t = timeit(lambda: api.check(api.int8_linear(stream, C.byref(lp))))
         report(f"INT8 linear {name} {Tq}x{K}x{Nn}", t, ops=2.0 * Tq * K * Nn, peak_ops=PEAK_I8)
         del a8, w8, o8
+    # ---- FP16 linear layers of a BERT-base FP16 encoder, B=128 x S=128 tokens ---------------------------
+    Th = 16384
+    for name, K, Nn, epi in (("feed-forward 1 + GELU", 768, 3072, capi.LINEAR_GELU),
+                             ("feed-forward 2", 3072, 768, capi.LINEAR_AFFINE)):
+        ah = torch.randn((Th, K), dtype=torch.float16, device="cuda")
+        wh = torch.randn((Nn, K), dtype=torch.float16, device="cuda") * (K ** -0.5)
+        al = torch.ones(Nn, device="cuda")
+        be = torch.zeros(Nn, device="cuda")
+        oh = torch.empty((Th, Nn), dtype=torch.float16, device="cuda")
+        hp = capi.Fp16LinearParams()
+        hp.a, hp.w, hp.alpha, hp.beta, hp.out = ah.data_ptr(), wh.data_ptr(), al.data_ptr(), be.data_ptr(), oh.data_ptr()
+        hp.T, hp.K, hp.N, hp.epilogue = Th, K, Nn, epi
+        t = timeit(lambda: api.check(api.fp16_linear(stream, C.byref(hp))))
+        report(f"FP16 linear {name} {Th}x{K}x{Nn}", t, ops=2.0 * Th * K * Nn, peak_ops=PEAK_F16)
+        del ah, wh, oh
     xh = torch.randn((Tq, 1024), dtype=torch.float16, device="cuda")
     x8 = torch.empty((32, Tq, 32), dtype=torch.int8, device="cuda")
     t = timeit(lambda: api.check(api.quantize_fp16_to_interleaved(stream, Tq, 1024, xh.data_ptr(), 0.03, x8.data_ptr())))

@@ -160,3 +160,53 @@ def test_bad_arguments_are_refused():
         assert "int8_linear" in api.last_error_str()
     p.T, p.K, p.N, p.epilogue, p.out_interleaved = 16, 64, 32, capi.LINEAR_RAW_INT32, 1
     assert api.int8_linear(None, C.byref(p)) != 0
+
+
+# ---- FP16 operands ---------------------------------------------------------------------------------
+
+def run_fp16(a, w, alpha, beta, gelu):
+    import torch
+    api = capi.api()
+    T, K = a.shape
+    N = w.shape[0]
+    da, dw, dal, dbe = dev(a), dev(w), dev(alpha), dev(beta)
+    out = dev_empty((T, N), np.float16, fill=-7)
+    p = capi.Fp16LinearParams()
+    p.a, p.w, p.alpha, p.beta, p.out = da.data_ptr(), dw.data_ptr(), dal.data_ptr(), dbe.data_ptr(), out.data_ptr()
+    p.T, p.K, p.N, p.epilogue = T, K, N, capi.LINEAR_GELU if gelu else capi.LINEAR_AFFINE
+    api.check(api.fp16_linear(torch.cuda.current_stream().cuda_stream, C.byref(p)))
+    torch.cuda.synchronize()
+    return host(out)
+
+
+@pytest.mark.parametrize("T,K,N", [(1, 32, 32), (77, 96, 64), (300, 768, 768), (519, 1024, 3072), (9000, 128, 1024),
+                                   (16500, 128, 1024)])
+@pytest.mark.parametrize("gelu", [False, True])
+def test_fp16_linear(T, K, N, gelu):
+    r = rng(61 + T)
+    a = (r.standard_normal((T, K)) * 0.5).astype(np.float16)
+    w = (r.standard_normal((N, K)) * (1.0 / np.sqrt(K))).astype(np.float16)
+    alpha = r.uniform(0.5, 1.5, N).astype(np.float32)
+    beta = (0.5 * r.standard_normal(N)).astype(np.float32)
+    got = run_fp16(a, w, alpha, beta, gelu)
+    ref = oracle.fp16_linear(a, w, alpha, beta, gelu)
+    assert_fp_close(got, ref, what="fp16 linear")
+    # and against binary64, so that the oracle's accumulation order is not what is being matched
+    y = (a.astype(np.float64) @ w.astype(np.float64).T) * alpha[None, :] + beta[None, :]
+    if gelu:
+        from scipy.special import erf
+        y = 0.5 * y * (1 + erf(y / np.sqrt(2)))
+    assert_fp_close(got, y, what="fp16 linear vs binary64")
+
+
+def test_fp16_linear_identity_is_exact_and_bad_arguments_are_refused():
+    api = capi.api()
+    a = (rng(3).standard_normal((50, 64))).astype(np.float16)
+    got = run_fp16(a, np.eye(64, dtype=np.float16), np.ones(64, np.float32), np.zeros(64, np.float32), False)
+    assert np.array_equal(got, a)
+    p = capi.Fp16LinearParams()
+    assert api.fp16_linear(None, C.byref(p)) != 0
+    d = dev(a)
+    p.a = p.w = p.alpha = p.beta = p.out = d.data_ptr()
+    p.T, p.K, p.N = 50, 48, 64
+    assert api.fp16_linear(None, C.byref(p)) != 0 and "fp16_linear" in api.last_error_str()

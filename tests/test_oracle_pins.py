@@ -585,3 +585,22 @@ def test_quantize_dequantize_reformat_closed_form():
     assert np.array_equal(back, (want.astype(np.float32) * scale).astype(np.float16))
     # quantise(dequantise(q)) is the identity when no value saturates the binary16 mantissa (|q| <= 128)
     assert np.array_equal(oracle.quantize_f16_interleave(back, float(scale)), q)
+
+
+def test_fp16_linear_against_float64():
+    from scipy.special import erf
+    r = rng(8)
+    T, K, N = 33, 96, 64
+    a = (r.standard_normal((T, K)) * 0.5).astype(np.float16)
+    w = (r.standard_normal((N, K)) * 0.2).astype(np.float16)
+    alpha = r.uniform(0.5, 1.5, N).astype(np.float32)
+    beta = r.standard_normal(N).astype(np.float32)
+    y = (a.astype(np.float64) @ w.astype(np.float64).T) * alpha[None, :] + beta[None, :]
+    got = oracle.fp16_linear(a, w, alpha, beta).astype(np.float64)
+    assert np.abs(got - y).max() <= 2e-3 + 1e-3 * np.abs(y).max()
+    g = 0.5 * y * (1 + erf(y / np.sqrt(2)))
+    got = oracle.fp16_linear(a, w, alpha, beta, gelu=True).astype(np.float64)
+    assert np.abs(got - g).max() <= 2e-3 + 1e-3 * np.abs(g).max()
+    # identity weights, unit scale, zero offset: the input comes back bit for bit
+    eye = np.eye(K, dtype=np.float16)
+    assert np.array_equal(oracle.fp16_linear(a, eye, np.ones(K, np.float32), np.zeros(K, np.float32)), a)
