@@ -125,16 +125,21 @@ def run_encoder(args, api, torch):
     segs = r.integers(0, 2, T).astype(np.int32)
     enc = Int8BertEncoder(cfg)
     enc.calibrate(ids, segs, cu)
-    enc.enqueue(ids, segs, cu)
+    want = enc.enqueue(ids, segs, cu)
+    # the timed pass is the native runner's (C++: plugin objects from the registry + the linear layers); the Python
+    # chain of the same calls stays available for comparison
+    step = enc.enqueue if args.python_runner else enc.enqueue_native
+    got = step()
     torch.cuda.synchronize()
+    assert torch.equal(got, want), "native runner and Python chain disagree"
 
-    clock_ramp(torch, enc.enqueue)
+    clock_ramp(torch, step)
     for _ in range(max(args.warmup, 1)):
-        enc.enqueue()
+        step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        enc.enqueue()
+        step()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
@@ -205,6 +210,7 @@ def run_encoder(args, api, torch):
                         "GEMM / SkipLayerNorm v7, dequantise; random-init weights, scales calibrated on the batch",
             "batch": args.batch, "max_seq_len": args.seqlen, "heads": N, "head_size": 64, "hidden": E, "ffn": F,
             "layers": cfg.layers, "tokens": T, "lengths": f"uniform[128,{args.seqlen}] seed {args.seed}",
+            "runner": "python" if args.python_runner else "native (trtamd_encoder_enqueue)",
         },
         "roofline": {
             "kernel": "int8_linear_persistent_kernel<true,true,true,GELU> (feed-forward 1)",
@@ -305,6 +311,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", choices=["encoder", "layer"], default="encoder")
     ap.add_argument("--layers", type=int, default=24, help="encoder workload only")
+    ap.add_argument("--python-runner", action="store_true",
+                    help="encoder workload: time the Python chain of plugin calls instead of the C++ runner")
     ap.add_argument("--batch", type=int, default=None, help="default 64 (layer) / 128 (encoder)")
     ap.add_argument("--seqlen", type=int, default=384)
     ap.add_argument("--seed", type=int, default=1)

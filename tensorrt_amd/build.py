@@ -36,7 +36,8 @@ def _hipcc() -> str:
 
 
 def sources() -> list[str]:
-    pats = ["*.hip", "*.cpp", os.path.join("plugin", "*.cpp"), os.path.join("plugin", "*.hip")]
+    pats = ["*.hip", "*.cpp", os.path.join("plugin", "*.cpp"), os.path.join("plugin", "*.hip"),
+            os.path.join("runtime", "*.cpp")]
     out: list[str] = []
     for p in pats:
         out += sorted(glob.glob(os.path.join(CSRC, p)))

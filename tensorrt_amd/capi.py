@@ -51,6 +51,27 @@ class Fp16LinearParams(C.Structure):
 
 LINEAR_AFFINE, LINEAR_GELU, LINEAR_RAW_INT32, LINEAR_AFFINE_FP16 = 0, 1, 2, 3
 
+
+class EncoderConfig(C.Structure):
+    """struct trtamd_encoder_config (include/trtamd_encoder_runtime.h)."""
+    _fields_ = [("hidden", i32), ("heads", i32), ("ffn", i32), ("layers", i32), ("vocab", i32), ("max_pos", i32),
+                ("type_vocab", i32), ("max_seqlen", i32)]
+
+
+class EncoderEmbedding(C.Structure):
+    _fields_ = [("beta", c_p), ("gamma", c_p), ("word", c_p), ("tok", c_p), ("pos", c_p), ("scale", f32)]
+
+
+class EncoderLinear(C.Structure):
+    _fields_ = [("w", c_p), ("alpha", c_p), ("beta", c_p)]
+
+
+class EncoderLayer(C.Structure):
+    _fields_ = [("qkv", EncoderLinear), ("proj", EncoderLinear), ("ffn1", EncoderLinear), ("ffn2", EncoderLinear),
+                ("ffn1_out_scale", f32),
+                ("ln1_gamma", c_p), ("ln1_beta", c_p), ("ln2_gamma", c_p), ("ln2_beta", c_p),
+                ("s_x", f32), ("s_qkv", f32), ("s_ctx", f32), ("s_ao", f32), ("s_h", f32), ("s_f", f32), ("s_out", f32)]
+
 _SIGS = {
     "trtamd_version": (C.c_int, []),
     "trtamd_last_error": (C.c_char_p, []),
@@ -85,6 +106,12 @@ _SIGS = {
     "trtamd_zero_padding_2d": (C.c_int, [c_p, i32, c_p, i32, i32, c_p]),
     "trtamd_int8_linear": (C.c_int, [c_p, C.POINTER(Int8LinearParams)]),
     "trtamd_fp16_linear": (C.c_int, [c_p, C.POINTER(Fp16LinearParams)]),
+    "trtamd_encoder_create": (c_p, [C.POINTER(EncoderConfig)]),
+    "trtamd_encoder_destroy": (None, [c_p]),
+    "trtamd_encoder_set_embedding": (C.c_int, [c_p, C.POINTER(EncoderEmbedding)]),
+    "trtamd_encoder_set_layer": (C.c_int, [c_p, i32, C.POINTER(EncoderLayer)]),
+    "trtamd_encoder_workspace_size": (C.c_size_t, [c_p, i32]),
+    "trtamd_encoder_enqueue": (C.c_int, [c_p, c_p, c_p, c_p, i32, i32, c_p, c_p, c_p]),
     "trtamd_int8_linear_to_interleaved": (C.c_int, [c_p, i32, i32, c_p, c_p]),
     "trtamd_int8_interleaved_to_linear": (C.c_int, [c_p, i32, i32, c_p, c_p]),
     "trtamd_quantize_fp16_to_interleaved": (C.c_int, [c_p, i32, i32, c_p, f32, c_p]),
@@ -95,7 +122,11 @@ _SIGS = {
 # Entry points declared in include/trtamd_encoder_ops.h.
 ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear", "trtamd_fp16_linear", "trtamd_int8_linear_to_interleaved", "trtamd_int8_interleaved_to_linear",
                        "trtamd_quantize_fp16_to_interleaved", "trtamd_dequantize_interleaved_to_fp16"]
-HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug" and k not in ENCODER_OPS_SYMBOLS]
+# Entry points declared in include/trtamd_encoder_runtime.h.
+ENCODER_RUNTIME_SYMBOLS = ["trtamd_encoder_create", "trtamd_encoder_destroy", "trtamd_encoder_set_embedding",
+                           "trtamd_encoder_set_layer", "trtamd_encoder_workspace_size", "trtamd_encoder_enqueue"]
+HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug" and k not in ENCODER_OPS_SYMBOLS
+                  and k not in ENCODER_RUNTIME_SYMBOLS]
 
 
 class TrtAmdError(RuntimeError):

@@ -1,0 +1,345 @@
+// Native runner of a built INT8 BERT encoder (include/trtamd_encoder_runtime.h): what a deserialised engine
+// holds (runtime-phase plugin objects from the registry, device weights, activation scales) and the
+// stream-ordered sequence of plugin enqueues and linear layers that executes it.  enqueue() only launches:
+// every device allocation happens in set_embedding / set_layer, the activations live in the caller's workspace.
+#include "plugin_common.h"
+#include "trtamd_encoder_runtime.h"
+
+#include "../host_utils.hpp"
+
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace trtamd
+{
+namespace runtime
+{
+namespace
+{
+
+using namespace trtamd::plugin;
+
+constexpr char const* kEMB = "CustomEmbLayerNormPluginDynamic";
+constexpr char const* kSKIP = "CustomSkipLayerNormPluginDynamic";
+constexpr char const* kQKV = "CustomQKVToContextPluginDynamic";
+
+struct PluginDeleter
+{
+    void operator()(IPluginV3* p) const
+    {
+        delete p;
+    }
+};
+using PluginPtr = std::unique_ptr<IPluginV3, PluginDeleter>;
+
+// Build-phase plugin -> serialised fields -> runtime-phase plugin, the round trip an engine file makes.
+PluginPtr makeRuntimePlugin(char const* name, char const* version, std::string const& layer,
+    std::vector<PluginField> const& fields)
+{
+    auto* creator = static_cast<IPluginCreatorV3One*>(getPluginRegistry()->getCreator(name, version, ""));
+    TRTAMD_VALIDATE_MSG(creator != nullptr, std::string(name) + " version " + version + " is not registered");
+    PluginFieldCollection fc{static_cast<int32_t>(fields.size()), fields.data()};
+    PluginPtr built(creator->createPlugin(layer.c_str(), &fc, TensorRTPhase::kBUILD));
+    TRTAMD_VALIDATE_MSG(built != nullptr, layer + ": createPlugin failed");
+    auto* rt = static_cast<IPluginV3OneRuntime*>(built->getCapabilityInterface(PluginCapabilityType::kRUNTIME));
+    PluginFieldCollection const* ser = rt->getFieldsToSerialize();
+    TRTAMD_VALIDATE_MSG(ser != nullptr, layer + ": getFieldsToSerialize failed");
+    PluginPtr runtime(creator->createPlugin(layer.c_str(), ser, TensorRTPhase::kRUNTIME));
+    TRTAMD_VALIDATE_MSG(runtime != nullptr, layer + ": runtime createPlugin failed");
+    return runtime;
+}
+
+IPluginV3OneRuntime* runtimeOf(PluginPtr const& p)
+{
+    return static_cast<IPluginV3OneRuntime*>(p->getCapabilityInterface(PluginCapabilityType::kRUNTIME));
+}
+
+PluginTensorDesc desc(std::initializer_list<int64_t> dims, DataType type, TensorFormat format, float scale)
+{
+    PluginTensorDesc d{};
+    d.dims.nbDims = static_cast<int32_t>(dims.size());
+    int32_t i = 0;
+    for (int64_t v : dims)
+    {
+        d.dims.d[i++] = v;
+    }
+    d.type = type;
+    d.format = format;
+    d.scale = scale;
+    return d;
+}
+
+// One INT8 fully-connected layer resident on the GPU: weights in the interleaved layout, folded scales.
+struct LinearLayer
+{
+    DeviceBuffer w, alpha, beta;
+    int32_t N{0}, K{0};
+
+    void load(trtamd_encoder_linear const& src, int32_t n, int32_t k)
+    {
+        TRTAMD_VALIDATE(src.w != nullptr && src.alpha != nullptr && src.beta != nullptr);
+        N = n;
+        K = k;
+        DeviceBuffer linear;
+        linear.upload(src.w, static_cast<size_t>(n) * k);
+        w.upload(src.w, static_cast<size_t>(n) * k); // allocation of the right size; overwritten below
+        checkKernelStatus(trtamd_int8_linear_to_interleaved(nullptr, n, k, linear.as<int8_t>(),
+                              static_cast<int8_t*>(w.get())),
+            "weight reformat");
+        TRTAMD_VALIDATE(hipStreamSynchronize(nullptr) == hipSuccess); // `linear` is freed on return
+        alpha.upload(src.alpha, sizeof(float) * n);
+        beta.upload(src.beta, sizeof(float) * n);
+    }
+
+    int run(hipStream_t stream, int8_t const* a, int8_t* out, int32_t tokens, int32_t epilogue, float outScale) const
+    {
+        trtamd_int8_linear_params p{};
+        p.a = a;
+        p.w = w.as<int8_t>();
+        p.alpha = alpha.as<float>();
+        p.beta = beta.as<float>();
+        p.out = out;
+        p.T = tokens;
+        p.K = K;
+        p.N = N;
+        p.a_interleaved = p.w_interleaved = p.out_interleaved = 1;
+        p.epilogue = epilogue;
+        p.out_scale = outScale;
+        return trtamd_int8_linear(stream, &p);
+    }
+};
+
+struct Layer
+{
+    LinearLayer qkv, proj, ffn1, ffn2;
+    PluginPtr attention, ln1, ln2;
+    float ffn1OutScale{1.f};
+    float sX{0}, sQkv{0}, sCtx{0}, sAo{0}, sH{0}, sF{0}, sOut{0};
+    bool set{false};
+};
+
+size_t align256(size_t n)
+{
+    return (n + 255) & ~size_t(255);
+}
+
+class Encoder
+{
+public:
+    explicit Encoder(trtamd_encoder_config const& c)
+        : mCfg(c)
+        , mLayers(static_cast<size_t>(c.layers))
+    {
+        TRTAMD_VALIDATE_MSG(c.hidden > 0 && c.heads > 0 && c.hidden == c.heads * 64,
+            "the INT8 interleaved attention plugin serves heads of 64 channels");
+        TRTAMD_VALIDATE(c.hidden % 64 == 0 && c.ffn % 64 == 0 && c.ffn > 0 && c.layers >= 0);
+        TRTAMD_VALIDATE(c.vocab > 0 && c.max_pos > 0 && c.type_vocab > 0 && c.max_seqlen > 0 && c.max_seqlen <= 512);
+    }
+
+    void setEmbedding(trtamd_encoder_embedding const& e)
+    {
+        TRTAMD_VALIDATE(e.beta && e.gamma && e.word && e.tok && e.pos && e.scale > 0.f);
+        int32_t const E = mCfg.hidden;
+        int32_t const fp16 = 1;
+        std::vector<PluginField> f{
+            {"bert_embeddings_layernorm_beta", e.beta, PluginFieldType::kFLOAT32, E},
+            {"bert_embeddings_layernorm_gamma", e.gamma, PluginFieldType::kFLOAT32, E},
+            {"bert_embeddings_word_embeddings", e.word, PluginFieldType::kFLOAT32, mCfg.vocab * E},
+            {"bert_embeddings_token_type_embeddings", e.tok, PluginFieldType::kFLOAT32, mCfg.type_vocab * E},
+            {"bert_embeddings_position_embeddings", e.pos, PluginFieldType::kFLOAT32, mCfg.max_pos * E},
+            {"output_fp16", &fp16, PluginFieldType::kINT32, 1}};
+        mEmbedding = makeRuntimePlugin(kEMB, "4", "embeddings", f);
+        mEmbScale = e.scale;
+    }
+
+    void setLayer(int32_t index, trtamd_encoder_layer const& l)
+    {
+        TRTAMD_VALIDATE_MSG(index >= 0 && index < mCfg.layers, "layer index out of range");
+        TRTAMD_VALIDATE(l.ln1_gamma && l.ln1_beta && l.ln2_gamma && l.ln2_beta);
+        TRTAMD_VALIDATE(l.s_x > 0 && l.s_qkv > 0 && l.s_ctx > 0 && l.s_ao > 0 && l.s_h > 0 && l.s_f > 0 && l.s_out > 0);
+        int32_t const E = mCfg.hidden, F = mCfg.ffn;
+        Layer& L = mLayers[static_cast<size_t>(index)];
+        L.qkv.load(l.qkv, 3 * E, E);
+        L.proj.load(l.proj, E, E);
+        L.ffn1.load(l.ffn1, F, E);
+        L.ffn2.load(l.ffn2, E, F);
+        L.ffn1OutScale = l.ffn1_out_scale;
+        std::string const tag = "l" + std::to_string(index);
+        float const dqProbs = 1.f / 127.f;
+        std::vector<PluginField> qf{{"hidden_size", &mCfg.hidden, PluginFieldType::kINT32, 1},
+            {"num_heads", &mCfg.heads, PluginFieldType::kINT32, 1}, {"dq_probs", &dqProbs, PluginFieldType::kFLOAT32, 1}};
+        L.attention = makeRuntimePlugin(kQKV, "6", tag + "_attention", qf);
+        auto ln = [&](char const* which, trtamd_half_t const* gamma, trtamd_half_t const* beta) {
+            std::vector<PluginField> f{{"beta", beta, PluginFieldType::kFLOAT16, E}, {"gamma", gamma, PluginFieldType::kFLOAT16, E}};
+            return makeRuntimePlugin(kSKIP, "7", tag + which, f);
+        };
+        L.ln1 = ln("_ln1", l.ln1_gamma, l.ln1_beta);
+        L.ln2 = ln("_ln2", l.ln2_gamma, l.ln2_beta);
+        L.sX = l.s_x;
+        L.sQkv = l.s_qkv;
+        L.sCtx = l.s_ctx;
+        L.sAo = l.s_ao;
+        L.sH = l.s_h;
+        L.sF = l.s_f;
+        L.sOut = l.s_out;
+        L.set = true;
+    }
+
+    // emb fp16 | x | qkv | ctx | ao | h | m | f | dummy | emb's second output
+    size_t workspaceSize(int32_t tokens) const
+    {
+        size_t const T = static_cast<size_t>(tokens > 0 ? tokens : 0);
+        size_t const E = static_cast<size_t>(mCfg.hidden), F = static_cast<size_t>(mCfg.ffn);
+        return align256(T * E * 2) + 5 * align256(T * E) + align256(3 * T * E) + align256(T * F)
+            + align256(sizeof(int32_t) * static_cast<size_t>(mCfg.max_seqlen)) + 256;
+    }
+
+    int enqueue(int32_t const* ids, int32_t const* segs, int32_t const* cu, int32_t batch, int32_t tokens,
+        void* workspace, trtamd_half_t* out, hipStream_t stream)
+    {
+        TRTAMD_VALIDATE_MSG(mEmbedding != nullptr, "set_embedding has not been called");
+        for (Layer const& L : mLayers)
+        {
+            TRTAMD_VALIDATE_MSG(L.set, "set_layer has not been called for every layer");
+        }
+        TRTAMD_VALIDATE(ids && segs && cu && workspace && out && batch > 0 && tokens > 0);
+        TRTAMD_VALIDATE_MSG((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "workspace must be 256-byte aligned");
+        int64_t const T = tokens, B = batch, E = mCfg.hidden, F = mCfg.ffn;
+
+        auto* base = static_cast<uint8_t*>(workspace);
+        auto carve = [&](size_t bytes) {
+            uint8_t* p = base;
+            base += align256(bytes);
+            return p;
+        };
+        auto* emb = reinterpret_cast<trtamd_half_t*>(carve(T * E * 2));
+        auto* x = reinterpret_cast<int8_t*>(carve(T * E));
+        auto* qkv = reinterpret_cast<int8_t*>(carve(3 * T * E));
+        auto* ctx = reinterpret_cast<int8_t*>(carve(T * E));
+        auto* ao = reinterpret_cast<int8_t*>(carve(T * E));
+        auto* h = reinterpret_cast<int8_t*>(carve(T * E));
+        auto* m = reinterpret_cast<int8_t*>(carve(T * F));
+        auto* f = reinterpret_cast<int8_t*>(carve(T * E));
+        auto* dummy = carve(sizeof(int32_t) * static_cast<size_t>(mCfg.max_seqlen)); // only its extent is read
+        auto* emb2 = carve(256);
+
+        auto run = [&](PluginPtr const& plugin, std::vector<PluginTensorDesc> const& in,
+                       std::vector<PluginTensorDesc> const& outDesc, std::vector<void const*> const& inputs,
+                       std::vector<void*> const& outputs, char const* what) {
+            IPluginV3OneRuntime* rt = runtimeOf(plugin);
+            int32_t st = rt->onShapeChange(in.data(), static_cast<int32_t>(in.size()), outDesc.data(),
+                static_cast<int32_t>(outDesc.size()));
+            if (st == 0)
+            {
+                st = rt->enqueue(in.data(), outDesc.data(), inputs.data(), outputs.data(), nullptr, stream);
+            }
+            TRTAMD_VALIDATE_MSG(st == 0, std::string(what) + " failed with status " + std::to_string(st));
+        };
+        auto const lin = TensorFormat::kLINEAR;
+        auto const il = TensorFormat::kCHW32;
+
+        run(mEmbedding,
+            {desc({T}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f),
+                desc({B + 1}, DataType::kINT32, lin, 1.f), desc({mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
+            {desc({T, E, 1, 1}, DataType::kHALF, lin, 1.f), desc({}, DataType::kINT32, lin, 1.f)}, {ids, segs, cu, dummy},
+            {emb, emb2}, "EmbLayerNorm");
+        checkKernelStatus(trtamd_quantize_fp16_to_interleaved(stream, tokens, mCfg.hidden, emb, mEmbScale, x), "quantise");
+
+        float lastScale = mEmbScale;
+        for (Layer const& L : mLayers)
+        {
+            checkKernelStatus(L.qkv.run(stream, x, qkv, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "QKV projection");
+            run(L.attention,
+                {desc({1, 3 * E, T, 1}, DataType::kINT8, il, L.sQkv), desc({B + 1}, DataType::kINT32, lin, 1.f),
+                    desc({mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
+                {desc({1, E, T, 1}, DataType::kINT8, il, L.sCtx)}, {qkv, cu, dummy}, {ctx}, "QKV-to-context");
+            checkKernelStatus(L.proj.run(stream, ctx, ao, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "output projection");
+            run(L.ln1, {desc({1, E, T, 1}, DataType::kINT8, il, L.sAo), desc({1, E, T, 1}, DataType::kINT8, il, L.sX)},
+                {desc({1, E, T, 1}, DataType::kINT8, il, L.sH)}, {ao, x}, {h}, "SkipLayerNorm 1");
+            checkKernelStatus(L.ffn1.run(stream, h, m, tokens, TRTAMD_LINEAR_GELU, L.ffn1OutScale), "feed-forward 1");
+            checkKernelStatus(L.ffn2.run(stream, m, f, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "feed-forward 2");
+            run(L.ln2, {desc({1, E, T, 1}, DataType::kINT8, il, L.sF), desc({1, E, T, 1}, DataType::kINT8, il, L.sH)},
+                {desc({1, E, T, 1}, DataType::kINT8, il, L.sOut)}, {f, h}, {x}, "SkipLayerNorm 2");
+            lastScale = L.sOut;
+        }
+        checkKernelStatus(trtamd_dequantize_interleaved_to_fp16(stream, tokens, mCfg.hidden, x, lastScale, out), "dequantise");
+        return TRTAMD_STATUS_SUCCESS;
+    }
+
+private:
+    trtamd_encoder_config mCfg;
+    PluginPtr mEmbedding;
+    float mEmbScale{0.f};
+    std::vector<Layer> mLayers;
+};
+
+template <typename Fn>
+int guarded(char const* what, Fn&& fn)
+{
+    try
+    {
+        return fn();
+    }
+    catch (std::exception const& e)
+    {
+        return set_error(TRTAMD_STATUS_FAILURE, "%s: %s", what, e.what());
+    }
+}
+
+} // namespace
+} // namespace runtime
+} // namespace trtamd
+
+using trtamd::runtime::Encoder;
+using trtamd::runtime::guarded;
+
+extern "C" trtamd_encoder_t trtamd_encoder_create(trtamd_encoder_config const* config)
+{
+    Encoder* enc = nullptr;
+    guarded("encoder_create", [&] {
+        TRTAMD_VALIDATE(config != nullptr);
+        enc = new Encoder(*config);
+        return 0;
+    });
+    return enc;
+}
+
+extern "C" void trtamd_encoder_destroy(trtamd_encoder_t encoder)
+{
+    delete static_cast<Encoder*>(encoder);
+}
+
+extern "C" int trtamd_encoder_set_embedding(trtamd_encoder_t encoder, trtamd_encoder_embedding const* embedding)
+{
+    return guarded("encoder_set_embedding", [&] {
+        TRTAMD_VALIDATE(encoder != nullptr && embedding != nullptr);
+        static_cast<Encoder*>(encoder)->setEmbedding(*embedding);
+        return 0;
+    });
+}
+
+extern "C" int trtamd_encoder_set_layer(trtamd_encoder_t encoder, int32_t index, trtamd_encoder_layer const* layer)
+{
+    return guarded("encoder_set_layer", [&] {
+        TRTAMD_VALIDATE(encoder != nullptr && layer != nullptr);
+        static_cast<Encoder*>(encoder)->setLayer(index, *layer);
+        return 0;
+    });
+}
+
+extern "C" size_t trtamd_encoder_workspace_size(trtamd_encoder_t encoder, int32_t max_tokens)
+{
+    return encoder ? static_cast<Encoder*>(encoder)->workspaceSize(max_tokens) : 0;
+}
+
+extern "C" int trtamd_encoder_enqueue(trtamd_encoder_t encoder, int32_t const* ids, int32_t const* segment_ids,
+    int32_t const* cu_seqlens, int32_t batch, int32_t tokens, void* workspace, trtamd_half_t* out,
+    trtamd_stream_t stream)
+{
+    return guarded("encoder_enqueue", [&] {
+        TRTAMD_VALIDATE(encoder != nullptr);
+        return static_cast<Encoder*>(encoder)->enqueue(ids, segment_ids, cu_seqlens, batch, tokens, workspace, out,
+            trtamd::as_stream(stream));
+    });
+}

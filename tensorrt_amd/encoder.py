@@ -348,6 +348,69 @@ class Int8BertEncoder:
         keep("out", b["out"])
         return b["out"]
 
+    # ---- the native runner ------------------------------------------------------------------------------
+    def build_native(self):
+        """Hands the built network (quantised weights, folded scales, calibrated activation scales) to the C++
+        runner of include/trtamd_encoder_runtime.h, which then owns its own plugin objects and device weights."""
+        if not self.calibrated:
+            raise RuntimeError("calibrate() first: the activation scales are not set")
+        api, cfg = self.api, self.cfg
+        c = capi.EncoderConfig(hidden=cfg.hidden, heads=cfg.heads, ffn=cfg.ffn, layers=cfg.layers, vocab=cfg.vocab,
+                               max_pos=cfg.max_pos, type_vocab=cfg.type_vocab, max_seqlen=cfg.max_seqlen)
+        h = api.encoder_create(C.byref(c))
+        if not h:
+            raise RuntimeError(f"trtamd_encoder_create: {api.last_error_str()}")
+        host = lambda a, dt: np.ascontiguousarray(a, dtype=dt)
+        ptr = lambda a: a.ctypes.data
+        w = self.emb_weights
+        keep = [host(w[k], np.float32) for k in ("beta", "gamma", "word", "tok", "pos")]
+        e = capi.EncoderEmbedding(*[ptr(a) for a in keep], self.s_emb)
+        api.check(api.encoder_set_embedding(h, C.byref(e)))
+        for i, L in enumerate(self.layers):
+            sc = L["scales"]
+            d = capi.EncoderLayer()
+            hold = []
+            for name in ("qkv", "proj", "ffn1", "ffn2"):
+                lin = L[name]
+                arrs = [host(lin.w_q, np.int8), host(lin.alpha_h, np.float32), host(lin.beta_h, np.float32)]
+                hold += arrs
+                setattr(d, name, capi.EncoderLinear(*[ptr(a) for a in arrs]))
+            d.ffn1_out_scale = L["ffn1"].out_scale
+            for field, key in (("ln1_gamma", "ln1_gamma"), ("ln1_beta", "ln1_beta"), ("ln2_gamma", "ln2_gamma"),
+                               ("ln2_beta", "ln2_beta")):
+                a = host(L[key], np.float16)
+                hold.append(a)
+                setattr(d, field, ptr(a))
+            d.s_x, d.s_qkv, d.s_ctx, d.s_ao = sc["x"], sc["qkv"], sc["ctx"], sc["ao"]
+            d.s_h, d.s_f, d.s_out = sc["h"], sc["f"], sc["out"]
+            api.check(api.encoder_set_layer(h, i, C.byref(d)))
+            del hold
+        self._native = h
+        self._native_ws = None
+        return h
+
+    def enqueue_native(self, ids=None, segs=None, cu=None):
+        """One forward pass through the C++ runner (same network, same scales); returns the FP16 output tensor."""
+        if getattr(self, "_native", None) is None:
+            self.build_native()
+        if ids is not None:
+            self._bind(ids, segs, cu)
+        torch, api, b = self.torch, self.api, self.buf
+        need = api.encoder_workspace_size(self._native, self.T)
+        if self._native_ws is None or self._native_ws.numel() < need:
+            self._native_ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
+        if "out_native" not in b or b["out_native"].shape[0] != self.T:
+            b["out_native"] = torch.empty((self.T, self.cfg.hidden), dtype=torch.float16, device="cuda")
+        api.check(api.encoder_enqueue(self._native, b["ids"].data_ptr(), b["segs"].data_ptr(), b["cu"].data_ptr(), self.B,
+                                      self.T, self._native_ws.data_ptr(), b["out_native"].data_ptr(), self.stream))
+        return b["out_native"]
+
+    def __del__(self):
+        h = getattr(self, "_native", None)
+        if h:
+            self.api.encoder_destroy(h)
+            self._native = None
+
     # ---- accounting ------------------------------------------------------------------------------------
     def gemm_ops(self) -> float:
         """Integer operations of the linear layers of one pass (2 per multiply-accumulate)."""

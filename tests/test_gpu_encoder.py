@@ -112,3 +112,23 @@ def test_output_dequantiser_and_repeatability(setup):
     again = enc.enqueue()
     torch.cuda.synchronize()
     assert np.array_equal(again.cpu().numpy(), out)
+
+
+def test_native_runner_matches_the_python_chain(setup):
+    """The C++ runner builds its own plugin objects and device weights from the same built network; its output
+    is the same bytes, on the calibration batch and on a batch of another shape."""
+    import torch
+    cfg, enc, ids, segs, cu, cap, out = setup
+    got = enc.enqueue_native(ids, segs, cu)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), out)
+    r = rng(17)
+    lens = np.array([3, 200, 64])
+    cu2 = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ids2 = r.integers(0, cfg.vocab, int(cu2[-1])).astype(np.int32)
+    segs2 = r.integers(0, 2, int(cu2[-1])).astype(np.int32)
+    want = enc.enqueue(ids2, segs2, cu2).cpu().numpy()
+    got = enc.enqueue_native(ids2, segs2, cu2)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    enc.enqueue(ids, segs, cu)   # leave the fixture's buffers as the other tests expect them

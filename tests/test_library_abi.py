@@ -44,6 +44,30 @@ def test_encoder_ops_header_symbols_exported(lib):
     assert sorted(capi.ENCODER_OPS_SYMBOLS) == names
 
 
+def test_encoder_runtime_header_symbols_exported(lib):
+    names = _declared("trtamd_encoder_runtime.h", "TRTAMD_API")
+    assert names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in trtamd_encoder_runtime.h but not exported"
+    assert sorted(capi.ENCODER_RUNTIME_SYMBOLS) == names
+
+
+def test_encoder_runtime_rejects_bad_configurations(lib):
+    a = capi.api()
+    bad = capi.EncoderConfig(hidden=1000, heads=16, ffn=4096, layers=2, vocab=10, max_pos=8, type_vocab=2, max_seqlen=128)
+    assert not a.encoder_create(ctypes.byref(bad))
+    assert "64 channels" in a.last_error_str()
+    ok = capi.EncoderConfig(hidden=128, heads=2, ffn=256, layers=1, vocab=10, max_pos=8, type_vocab=2, max_seqlen=128)
+    h = a.encoder_create(ctypes.byref(ok))
+    assert h
+    # emb fp16 + five hidden-wide INT8 tensors + QKV + FFN intermediate + the two small extras, each 256-byte aligned
+    assert a.encoder_workspace_size(h, 100) == 25600 + 5 * 12800 + 38400 + 25600 + 512 + 256
+    assert a.encoder_enqueue(h, None, None, None, 1, 100, None, None, None) != 0
+    assert "set_embedding" in a.last_error_str()
+    assert a.encoder_set_layer(h, 3, ctypes.byref(capi.EncoderLayer())) != 0
+    a.encoder_destroy(h)
+
+
 def test_plugin_c_header_symbols_exported(lib):
     from tensorrt_amd import plugin
     names = _declared("trtamd_plugin_c.h", "TRTAMD_PLUGIN_API")
