@@ -250,7 +250,57 @@ def run_encoder(args, api, torch):
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_encoder(enc, cu, ms_budget_s=20.0)
+        out["cpu_baseline_fp32_library"] = cpu_baseline_torch(enc, cu, lens, torch)
     return out
+
+
+def cpu_baseline_torch(enc, cu, lens, torch, budget_s=8.0):
+    """What a CPU inference library does with the same network: the de-quantised FP32 subgraph of one layer
+    (MatMul + bias, per-sequence softmax attention, Add + LayerNormalization, erf GELU) through torch's CPU
+    kernels on every host core, scaled to the number of layers.  The reference's own CPU route is this graph in
+    onnxruntime (tools/Polygraphy/polygraphy/backend/onnxrt/loader.py:74-85), which is not installed here."""
+    cores = len(os.sched_getaffinity(0))
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    cfg = enc.cfg
+    E, N = cfg.hidden, cfg.heads
+    nseq = min(16, len(lens))
+    T = int(cu[nseq])
+    L = enc.layers[0]
+    W = {k: torch.from_numpy(L[k].w_q.astype(np.float32) * L[k].s_w[:, None]) for k in ("qkv", "proj", "ffn1", "ffn2")}
+    Bv = {k: torch.from_numpy(L[k].bias) for k in W}
+    g1, b1 = (torch.from_numpy(L[k].astype(np.float32)) for k in ("ln1_gamma", "ln1_beta"))
+    g2, b2 = (torch.from_numpy(L[k].astype(np.float32)) for k in ("ln2_gamma", "ln2_beta"))
+    x = torch.randn(T, E)
+    F = torch.nn.functional
+
+    def layer(x):
+        qkv = F.linear(x, W["qkv"], Bv["qkv"])
+        ctx = torch.empty(T, E)
+        for b in range(nseq):
+            lo, hi = int(cu[b]), int(cu[b + 1])
+            q, k, v = (qkv[lo:hi, i * E:(i + 1) * E].reshape(hi - lo, N, 64).transpose(0, 1) for i in range(3))
+            o = torch.softmax(q @ k.transpose(1, 2) * 0.125, -1) @ v
+            ctx[lo:hi] = o.transpose(0, 1).reshape(hi - lo, E)
+        h = F.layer_norm(F.linear(ctx, W["proj"], Bv["proj"]) + x, (E,), g1, b1, 1e-12)
+        m = F.gelu(F.linear(h, W["ffn1"], Bv["ffn1"]))
+        return F.layer_norm(F.linear(m, W["ffn2"], Bv["ffn2"]) + h, (E,), g2, b2, 1e-12)
+
+    with torch.no_grad():
+        layer(x)
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            layer(x)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el > budget_s:
+                break
+    per_layer = el / reps
+    return {"value": round(nseq / (per_layer * cfg.layers), 3), "unit": "sequences/s", "cores": threads,
+            "kind": "torch-CPU FP32 fallback (onnxruntime unavailable)",
+            "sample": f"{reps} pass(es) of ONE de-quantised FP32 layer through torch CPU kernels over the first {nseq} "
+                      f"sequences ({T} tokens) in {el:.1f} s, scaled by {cfg.layers} layers"}
 
 
 def cpu_baseline_encoder(enc, cu, ms_budget_s=20.0):
