@@ -65,7 +65,10 @@ __device__ inline bool locate_token(int64_t wave, int B, int S, int32_t const* c
     return true;
 }
 
-template <typename T, int NV, int MODE>
+// TPW consecutive token slots per wavefront.  gamma and beta are fetched once per wavefront (converted to T and
+// back, as the reference does per element) instead of once per token: at TPW = 1 they are two thirds of the
+// bytes a token pulls through the vector cache.
+template <typename T, int NV, int MODE, int TPW>
 __global__ __launch_bounds__(kBlock) void embln_kernel(int const ld, int const B, int const S,
     int32_t const* __restrict__ inputIds, int32_t const* __restrict__ tokenIds, int32_t const* __restrict__ cuSeqlens,
     float const* __restrict__ beta, float const* __restrict__ gamma, T const* __restrict__ wordEmb,
@@ -76,92 +79,108 @@ __global__ __launch_bounds__(kBlock) void embln_kernel(int const ld, int const B
     int const lane = threadIdx.x & (kWaveSize - 1);
     int64_t const wave
         = __builtin_amdgcn_readfirstlane((int) ((int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)));
-    int64_t tokenIdx;
-    int pos;
-    if (!locate_token<MODE>(wave, B, S, cuSeqlens, tokenIdx, pos))
-    {
-        return;
-    }
-    int const wordId = __builtin_amdgcn_readfirstlane(inputIds[tokenIdx]);
-    int const tokId = __builtin_amdgcn_readfirstlane(tokenIds[tokenIdx]);
-    bool const inRange = wordId >= 0 && wordId < wordSize && tokId >= 0 && tokId < tokSize;
     int const nvec = ld / VPT;
 
-    Vec16<T> w[NV], t[NV], p[NV];
+    // gamma/beta take the output type first: `const R g(gamma[i])`, common.cuh:275-276
+    float gk[NV][VPT], bk[NV][VPT];
 #pragma unroll
     for (int j = 0; j < NV; ++j)
     {
         int const vi = lane + kWaveSize * j;
-        bool const ok = vi < nvec && inRange;
-        w[j].u = ok ? *reinterpret_cast<u32x4 const*>(wordEmb + (int64_t) wordId * ld + vi * VPT) : u32x4{0, 0, 0, 0};
-        t[j].u = ok ? *reinterpret_cast<u32x4 const*>(tokEmb + (int64_t) tokId * ld + vi * VPT) : u32x4{0, 0, 0, 0};
-        p[j].u = ok ? *reinterpret_cast<u32x4 const*>(posEmb + (int64_t) pos * ld + vi * VPT) : u32x4{0, 0, 0, 0};
+        bool const ok = vi < nvec;
+#pragma unroll
+        for (int q = 0; q < VPT / 4; ++q)
+        {
+            f32x4 const g4 = ok ? *reinterpret_cast<f32x4 const*>(gamma + vi * VPT + q * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+            f32x4 const b4 = ok ? *reinterpret_cast<f32x4 const*>(beta + vi * VPT + q * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+            {
+                gk[j][q * 4 + e] = (float) (T) g4[e];
+                bk[j][q * 4 + e] = (float) (T) b4[e];
+            }
+        }
     }
 
-    float v[NV][VPT];
-    float sum = 0.f, cnt = 0.f;
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
+#pragma unroll 1
+    for (int it = 0; it < TPW; ++it)
     {
-        bool const ok = lane + kWaveSize * j < nvec;
-        Vec16<T> pre;
-#pragma unroll
-        for (int k = 0; k < VPT; ++k)
+        int64_t tokenIdx;
+        int pos;
+        if (!locate_token<MODE>(wave * TPW + it, B, S, cuSeqlens, tokenIdx, pos))
         {
-            T const s = (w[j].e[k] + t[j].e[k]) + p[j].e[k];
-            pre.e[k] = s;
-            v[j][k] = (float) s;
-            sum += ok ? v[j][k] : 0.f;
+            continue;
         }
-        cnt += ok ? (float) VPT : 0.f;
-        if (MODE == kMTRON && ok)
+        int const wordId = __builtin_amdgcn_readfirstlane(inputIds[tokenIdx]);
+        int const tokId = __builtin_amdgcn_readfirstlane(tokenIds[tokenIdx]);
+        bool const inRange = wordId >= 0 && wordId < wordSize && tokId >= 0 && tokId < tokSize;
+
+        Vec16<T> w[NV], t[NV], p[NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
         {
-            *reinterpret_cast<u32x4*>(skipOut + tokenIdx * ld + (int64_t) (lane + kWaveSize * j) * VPT) = pre.u;
+            int const vi = lane + kWaveSize * j;
+            bool const ok = vi < nvec && inRange;
+            w[j].u = ok ? *reinterpret_cast<u32x4 const*>(wordEmb + (int64_t) wordId * ld + vi * VPT) : u32x4{0, 0, 0, 0};
+            t[j].u = ok ? *reinterpret_cast<u32x4 const*>(tokEmb + (int64_t) tokId * ld + vi * VPT) : u32x4{0, 0, 0, 0};
+            p[j].u = ok ? *reinterpret_cast<u32x4 const*>(posEmb + (int64_t) pos * ld + vi * VPT) : u32x4{0, 0, 0, 0};
         }
-    }
-    Welford st;
-    st.n = cnt;
-    st.mean = cnt > 0.f ? sum / cnt : 0.f;
-    st.m2 = 0.f;
+
+        float v[NV][VPT];
+        float sum = 0.f, cnt = 0.f;
 #pragma unroll
-    for (int j = 0; j < NV; ++j)
-    {
-        bool const ok = lane + kWaveSize * j < nvec;
-#pragma unroll
-        for (int k = 0; k < VPT; ++k)
+        for (int j = 0; j < NV; ++j)
         {
-            float const dlt = v[j][k] - st.mean;
-            st.m2 += ok ? dlt * dlt : 0.f;
-        }
-    }
-    st = group_welford<kWaveSize>(st);
-    float const mu = st.mean;
-    // No epsilon (plugin/common/common.cuh:269).  Ids out of range leave the reference's row
-    // undefined; here such a row is the LayerNorm of zeros with rsigma forced to 0, i.e. beta.
-    float const rsigma = inRange ? rsqrtf(st.m2 / (float) ld) : 0.f;
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
-    {
-        int const vi = lane + kWaveSize * j;
-        if (vi < nvec)
-        {
-            f32x4 gq[VPT / 4], bq[VPT / 4];
-#pragma unroll
-            for (int q = 0; q < VPT / 4; ++q)
-            {
-                gq[q] = *reinterpret_cast<f32x4 const*>(gamma + vi * VPT + q * 4);
-                bq[q] = *reinterpret_cast<f32x4 const*>(beta + vi * VPT + q * 4);
-            }
-            Vec16<T> y;
+            bool const ok = lane + kWaveSize * j < nvec;
+            Vec16<T> pre;
 #pragma unroll
             for (int k = 0; k < VPT; ++k)
             {
-                // gamma/beta take the output type first: `const R g(gamma[i])`, common.cuh:275-276
-                float const gk = (float) (T) gq[k >> 2][k & 3];
-                float const bk = (float) (T) bq[k >> 2][k & 3];
-                y.e[k] = (T) (gk * (v[j][k] - mu) * rsigma + bk);
+                T const s = (w[j].e[k] + t[j].e[k]) + p[j].e[k];
+                pre.e[k] = s;
+                v[j][k] = (float) s;
+                sum += ok ? v[j][k] : 0.f;
             }
-            *reinterpret_cast<u32x4*>(output + tokenIdx * ld + (int64_t) vi * VPT) = y.u;
+            cnt += ok ? (float) VPT : 0.f;
+            if (MODE == kMTRON && ok)
+            {
+                *reinterpret_cast<u32x4*>(skipOut + tokenIdx * ld + (int64_t) (lane + kWaveSize * j) * VPT) = pre.u;
+            }
+        }
+        Welford st;
+        st.n = cnt;
+        st.mean = cnt > 0.f ? sum / cnt : 0.f;
+        st.m2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            bool const ok = lane + kWaveSize * j < nvec;
+#pragma unroll
+            for (int k = 0; k < VPT; ++k)
+            {
+                float const dlt = v[j][k] - st.mean;
+                st.m2 += ok ? dlt * dlt : 0.f;
+            }
+        }
+        st = group_welford<kWaveSize>(st);
+        float const mu = st.mean;
+        // No epsilon (plugin/common/common.cuh:269).  Ids out of range leave the reference's row
+        // undefined; here such a row is the LayerNorm of zeros with rsigma forced to 0, i.e. beta.
+        float const rsigma = inRange ? rsqrtf(st.m2 / (float) ld) : 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            int const vi = lane + kWaveSize * j;
+            if (vi < nvec)
+            {
+                Vec16<T> y;
+#pragma unroll
+                for (int k = 0; k < VPT; ++k)
+                {
+                    y.e[k] = (T) (gk[j][k] * (v[j][k] - mu) * rsigma + bk[j][k]);
+                }
+                *reinterpret_cast<u32x4*>(output + tokenIdx * ld + (int64_t) vi * VPT) = y.u;
+            }
         }
     }
 }
@@ -246,9 +265,21 @@ int emb_layer_norm(hipStream_t stream, int32_t ld, int32_t B, int32_t S, int32_t
         && aligned16(output) && aligned16(beta) && aligned16(gamma) && (MODE != kMTRON || aligned16(skipOut));
     int const nv = vec_ok ? ceil_div(ld / VPT, kWaveSize) : 0;
     dim3 const grid((unsigned) ceil_div<int64_t>((int64_t) S * B, kWavesPerBlock));
+    // several tokens per wavefront once there are enough token slots to keep every SIMD busy anyway
+    int64_t const slots = (int64_t) S * B;
+    bool const multi = slots >= 65536;
+    dim3 const grid4((unsigned) ceil_div<int64_t>(ceil_div<int64_t>(slots, 4), kWavesPerBlock));
 #define TRTAMD_EMB_LAUNCH(NVV)                                                                                         \
-    hipLaunchKernelGGL((embln_kernel<T, NVV, MODE>), grid, dim3(kBlock), 0, stream, ld, B, S, inputIds, tokenIds,        \
-        cuSeqlens, beta, gamma, wordEmb, posEmb, tokEmb, wordSize, tokSize, output, skipOut)
+    if (multi)                                                                                                         \
+    {                                                                                                                  \
+        hipLaunchKernelGGL((embln_kernel<T, NVV, MODE, 4>), grid4, dim3(kBlock), 0, stream, ld, B, S, inputIds,          \
+            tokenIds, cuSeqlens, beta, gamma, wordEmb, posEmb, tokEmb, wordSize, tokSize, output, skipOut);            \
+    }                                                                                                                  \
+    else                                                                                                               \
+    {                                                                                                                  \
+        hipLaunchKernelGGL((embln_kernel<T, NVV, MODE, 1>), grid, dim3(kBlock), 0, stream, ld, B, S, inputIds,           \
+            tokenIds, cuSeqlens, beta, gamma, wordEmb, posEmb, tokEmb, wordSize, tokSize, output, skipOut);            \
+    }
     if (vec_ok && nv == 1)
     {
         TRTAMD_EMB_LAUNCH(1);
