@@ -124,20 +124,120 @@ __device__ inline int frag_offset(int row, int half)
     return row * 32 + ((half ^ ((row >> 3) & 1)) << 4);
 }
 
-// Epilogue of one workgroup tile.  Accumulator register v of a 32x32 tile is token l%32, channel
-// 8*(v/4) + 4*(l/32) + v%4: four groups of four consecutive channels.  For the INT8 outputs the two lanes
-// that share a token trade two packed dwords (v_permlane32_swap), after which lane l holds the 16
-// consecutive channels 16*(l/32)..+15 and stores them with one 16-byte write.
+// Epilogue of one 32 x 32 accumulator block whose first channel is c0 (sAlpha / sBeta point at that channel's
+// entry) and first token tb.  Accumulator register v is token l%32, channel 8*(v/4) + 4*(l/32) + v%4: four groups
+// of four consecutive channels.  For the INT8 outputs the two lanes that share a token trade two packed dwords
+// (v_permlane32_swap), after which lane l holds the 16 consecutive channels 16*(l/32)..+15 and stores them with
+// one 16-byte write.
+template <bool IL_OUT, int EPI>
+__device__ __forceinline__ void store_block(
+    LinearArgs const& p, AccT<EPI> const& acc, int const c0, int const tb, float const* sAlpha, float const* sBeta)
+{
+    int const lane = threadIdx.x & 63;
+    int const hi = lane >> 5;
+    int const t = tb + (lane & 31);
+    bool const live = t < p.T;
+    f32x4 al[4], be[4];
+    if constexpr (EPI != kRAW)
+    {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+        {
+            al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + 8 * g + 4 * hi);
+            be[g] = *reinterpret_cast<f32x4 const*>(sBeta + 8 * g + 4 * hi);
+        }
+    }
+    if constexpr (EPI == kRAW)
+    {
+        if (live)
+        {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                i32x4 const v = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+                *reinterpret_cast<i32x4*>(static_cast<int32_t*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi) = v;
+            }
+        }
+    }
+    else if constexpr (EPI >= kF16_AFFINE)
+    {
+        if (live)
+        {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                f16x4 h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    float const y = fmaf(acc[4 * g + e], al[g][e], be[g][e]);
+                    h[e] = (f16) (EPI == kF16_GELU ? gelu_erf(y) : y);
+                }
+                *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi) = h;
+            }
+        }
+    }
+    else if constexpr (EPI == kHALF)
+    {
+        if (live)
+        {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                f16x4 h;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    h[e] = (f16) fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
+                }
+                *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi) = h;
+            }
+        }
+    }
+    else
+    {
+        int d[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+        {
+            uint32_t b[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+            {
+                float y = fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
+                if constexpr (EPI == kGELU)
+                {
+                    // one rounding of gelu * scale + 1.5*2^23: the sum's low bits are the integer
+                    b[e] = clamp_sat8_bits(fmaf(gelu_erf(y), p.qOut, kRoundMagic));
+                }
+                else
+                {
+                    b[e] = round_sat8_bits(y);
+                }
+            }
+            d[g] = (int) low_bytes(b[0], b[1], b[2], b[3]);
+        }
+        // lanes l < 32 hold channels [0-3][8-11][16-19][24-27], lanes l+32 the gaps
+        auto const s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+        auto const s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+        i32x4 const packed = {(int) s02[0], (int) s02[1], (int) s13[0], (int) s13[1]};
+        if (live)
+        {
+            int const c = c0 + 16 * hi;
+            size_t const o = IL_OUT ? ((size_t) (c >> 5) * p.T + t) * 32 + (c & 31) : (size_t) t * p.N + c;
+            *reinterpret_cast<i32x4*>(static_cast<int8_t*>(p.out) + o) = packed;
+        }
+    }
+}
+
+// Epilogue of one workgroup tile.
 template <int WM, int WN, int MT, int NT, bool IL_OUT, int EPI>
 __device__ __forceinline__ void store_tile(LinearArgs const& p, AccT<EPI> const (&acc)[MT][NT], int const n0, int const t0,
     float const* sAlpha, float const* sBeta)
 {
-    int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const wm = wave / WN;
     int const wn = wave % WN;
-    int const col32 = lane & 31;
-    int const hi = lane >> 5;
 #pragma unroll
     for (int i = 0; i < MT; ++i)
     {
@@ -146,107 +246,10 @@ __device__ __forceinline__ void store_tile(LinearArgs const& p, AccT<EPI> const 
         {
             break;
         }
-        f32x4 al[4], be[4];
-        if constexpr (EPI != kRAW)
-        {
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-            {
-                al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + cl + 8 * g + 4 * hi);
-                be[g] = *reinterpret_cast<f32x4 const*>(sBeta + cl + 8 * g + 4 * hi);
-            }
-        }
 #pragma unroll
         for (int j = 0; j < NT; ++j)
         {
-            int const t = t0 + (wn * NT + j) * 32 + col32;
-            bool const live = t < p.T;
-            if constexpr (EPI == kRAW)
-            {
-                if (live)
-                {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                    {
-                        i32x4 const v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                            acc[i][j][4 * g + 3]};
-                        *reinterpret_cast<i32x4*>(
-                            static_cast<int32_t*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
-                            = v;
-                    }
-                }
-            }
-            else if constexpr (EPI >= kF16_AFFINE)
-            {
-                if (live)
-                {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                    {
-                        f16x4 h;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                        {
-                            float const y = fmaf(acc[i][j][4 * g + e], al[g][e], be[g][e]);
-                            h[e] = (f16) (EPI == kF16_GELU ? gelu_erf(y) : y);
-                        }
-                        *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
-                            = h;
-                    }
-                }
-            }
-            else if constexpr (EPI == kHALF)
-            {
-                if (live)
-                {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                    {
-                        f16x4 h;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                        {
-                            h[e] = (f16) fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
-                        }
-                        *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + n0 + cl + 8 * g + 4 * hi)
-                            = h;
-                    }
-                }
-            }
-            else
-            {
-                int d[4];
-#pragma unroll
-                for (int g = 0; g < 4; ++g)
-                {
-                    uint32_t b[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                    {
-                        float y = fmaf((float) acc[i][j][4 * g + e], al[g][e], be[g][e]);
-                        if constexpr (EPI == kGELU)
-                        {
-                            // one rounding of gelu * scale + 1.5*2^23: the sum's low bits are the integer
-                            b[e] = clamp_sat8_bits(fmaf(gelu_erf(y), p.qOut, kRoundMagic));
-                        }
-                        else
-                        {
-                            b[e] = round_sat8_bits(y);
-                        }
-                    }
-                    d[g] = (int) low_bytes(b[0], b[1], b[2], b[3]);
-                }
-                // lanes l < 32 hold channels [0-3][8-11][16-19][24-27], lanes l+32 the gaps
-                auto const s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-                auto const s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-                i32x4 const packed = {(int) s02[0], (int) s02[1], (int) s13[0], (int) s13[1]};
-                if (live)
-                {
-                    int const c = n0 + cl + 16 * hi;
-                    size_t const o = IL_OUT ? ((size_t) (c >> 5) * p.T + t) * 32 + (c & 31) : (size_t) t * p.N + c;
-                    *reinterpret_cast<i32x4*>(static_cast<int8_t*>(p.out) + o) = packed;
-                }
-            }
+            store_block<IL_OUT, EPI>(p, acc[i][j], n0 + cl, t0 + (wn * NT + j) * 32, sAlpha + cl, sBeta + cl);
         }
     }
 }
