@@ -233,6 +233,10 @@ def run_encoder(args, api, torch):
             "traffic": ENC_MHA_TRAFFIC_BYTES if default_workload else None,
             "avg_launch_us": table["attention"]["avg_launch_us"],
             "algorithmic_ops_per_launch": ops["attention"][1],
+            # its arithmetic intensity (ops per byte of q, k, v and context) is below the machine's ridge of
+            # 625 INT8 ops per HBM byte, so the HBM figure is the nearer roof
+            "algorithmic_bytes_per_launch": 4 * T * E,
+            "hbm_frac": round(4 * T * E / (table["attention"]["avg_launch_us"] * 1e-6) / PEAK_HBM, 4),
         },
         "roofline_skipln": {
             "kernel": "skipln_interleaved_kernel<32,8,32,false>",
