@@ -132,6 +132,16 @@ def run_encoder(args, api, torch):
     got = step()
     torch.cuda.synchronize()
     assert torch.equal(got, want), "native runner and Python chain disagree"
+    if args.graph and not args.python_runner:
+        # the native enqueue only launches kernels: record one pass, time its replays
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            got = enc.enqueue_native(stream=torch.cuda.current_stream().cuda_stream)
+        step = graph.replay
+        got.zero_()
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), "graph replay and eager pass disagree"
 
     clock_ramp(torch, step)
     for _ in range(max(args.warmup, 1)):
@@ -210,7 +220,8 @@ def run_encoder(args, api, torch):
                         "GEMM / SkipLayerNorm v7, dequantise; random-init weights, scales calibrated on the batch",
             "batch": args.batch, "max_seq_len": args.seqlen, "heads": N, "head_size": 64, "hidden": E, "ffn": F,
             "layers": cfg.layers, "tokens": T, "lengths": f"uniform[128,{args.seqlen}] seed {args.seed}",
-            "runner": "python" if args.python_runner else "native (trtamd_encoder_enqueue)",
+            "runner": "python" if args.python_runner else "native (trtamd_encoder_enqueue)"
+                      + (", replayed from a captured graph" if args.graph else ""),
         },
         "roofline": {
             "kernel": "int8_linear_persistent_kernel<true,true,true,GELU> (feed-forward 1)",
@@ -365,6 +376,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", choices=["encoder", "layer"], default="encoder")
     ap.add_argument("--layers", type=int, default=24, help="encoder workload only")
+    ap.add_argument("--graph", action="store_true",
+                    help="encoder workload: record the native runner's pass into a graph and time its replays")
     ap.add_argument("--python-runner", action="store_true",
                     help="encoder workload: time the Python chain of plugin calls instead of the C++ runner")
     ap.add_argument("--batch", type=int, default=None, help="default 64 (layer) / 128 (encoder)")

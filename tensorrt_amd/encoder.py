@@ -389,8 +389,10 @@ class Int8BertEncoder:
         self._native_ws = None
         return h
 
-    def enqueue_native(self, ids=None, segs=None, cu=None):
-        """One forward pass through the C++ runner (same network, same scales); returns the FP16 output tensor."""
+    def enqueue_native(self, ids=None, segs=None, cu=None, stream=None):
+        """One forward pass through the C++ runner (same network, same scales); returns the FP16 output tensor.
+        `stream` (a raw stream handle) overrides the stream the encoder was built on, e.g. a stream under graph
+        capture: the call only launches kernels, so it can be recorded and replayed."""
         if getattr(self, "_native", None) is None:
             self.build_native()
         if ids is not None:
@@ -402,7 +404,8 @@ class Int8BertEncoder:
         if "out_native" not in b or b["out_native"].shape[0] != self.T:
             b["out_native"] = torch.empty((self.T, self.cfg.hidden), dtype=torch.float16, device="cuda")
         api.check(api.encoder_enqueue(self._native, b["ids"].data_ptr(), b["segs"].data_ptr(), b["cu"].data_ptr(), self.B,
-                                      self.T, self._native_ws.data_ptr(), b["out_native"].data_ptr(), self.stream))
+                                      self.T, self._native_ws.data_ptr(), b["out_native"].data_ptr(),
+                                      self.stream if stream is None else stream))
         return b["out_native"]
 
     def __del__(self):

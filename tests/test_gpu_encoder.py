@@ -132,3 +132,32 @@ def test_native_runner_matches_the_python_chain(setup):
     torch.cuda.synchronize()
     assert np.array_equal(got.cpu().numpy(), want)
     enc.enqueue(ids, segs, cu)   # leave the fixture's buffers as the other tests expect them
+
+
+def test_native_runner_replays_from_a_captured_graph(setup):
+    """enqueue launches kernels only (no allocation, copy, memset or synchronisation), so a caller can record it
+    into a graph.  Every replay is checked, with eager work on the same buffers between the replays."""
+    import torch
+    cfg, enc, ids, segs, cu, cap, out = setup
+    first = enc.enqueue_native(ids, segs, cu)
+    torch.cuda.synchronize()
+    assert np.array_equal(first.cpu().numpy(), out)
+    r = rng(23)
+    ids2 = r.integers(0, cfg.vocab, ids.size).astype(np.int32)
+    want2 = enc.enqueue_native(ids2, segs, cu).cpu().numpy()
+    enc.enqueue_native(ids, segs, cu)
+    torch.cuda.synchronize()
+    assert not np.array_equal(want2, out)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        result = enc.enqueue_native(stream=torch.cuda.current_stream().cuda_stream)
+    d_ids = enc.buf["ids"]
+    for k, (tokens, want) in enumerate([(ids, out), (ids2, want2), (ids, out), (ids2, want2)]):
+        d_ids.copy_(torch.from_numpy(tokens))          # eager: new inputs in place
+        result.fill_(float("nan"))                     # eager: the previous result is gone
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(result.cpu().numpy(), want), f"replay {k}"
+    enc.enqueue(ids, segs, cu)   # leave the fixture's buffers as the other tests expect them
