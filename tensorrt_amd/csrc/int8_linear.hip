@@ -723,7 +723,18 @@ int launch_shape(hipStream_t stream, LinearArgs a)
     int const nbmBig = ceil_div(a.N, kBig);
     int64_t const bigTiles = (int64_t) nbmBig * (a.T / kBig);
     int const cus = num_cus();
-    a.tokMain = (int) ((bigTiles / cus) * cus / nbmBig);
+    // ... plus a last partial round when it would occupy more than `partial` per cent of the CUs: in 128 x 128
+    // tiles that remainder needs three rounds or more, which take longer than one round of large tiles
+    static int const partial = [] {
+        char const* e = getenv("TRTAMD_LINEAR_PARTIAL_ROUND");
+        return e ? atoi(e) : 50;
+    }();
+    int64_t roundedTiles = (bigTiles / cus) * cus;
+    if ((bigTiles - roundedTiles) * 100 > (int64_t) partial * cus)
+    {
+        roundedTiles = bigTiles;
+    }
+    a.tokMain = (int) (roundedTiles / nbmBig);
     a.mainTiles = a.tokMain * nbmBig;
     constexpr int kMaxPanel = 8; // 8 x 256 channels x K = 1024 of weights is half of an XCD's 4 MB L2
     a.panel = 1;

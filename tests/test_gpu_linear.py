@@ -113,9 +113,12 @@ def test_affine_fp16(T, K, N):
     assert_fp_close(got, ref, what="fp16 output")
 
 
-@pytest.mark.parametrize("T,K,N", [(8229, 128, 3072), (16500, 64, 1024), (70000, 64, 256)])
+@pytest.mark.parametrize("T,K,N", [(8229, 128, 3072), (16500, 64, 1024), (70000, 64, 256), (9600, 128, 1024),
+                                   (28165, 128, 1024)])
 def test_large_problems_mix_both_tile_sizes(T, K, N):
-    """Enough 256 x 256 tiles for whole rounds of the chip, plus a remainder in 128 x 128 tiles."""
+    """Enough 256 x 256 tiles for whole rounds of the chip, plus a remainder in 128 x 128 tiles.  The last two
+    sizes leave more than half a round of large tiles, which then runs as a partial round (one with no whole
+    round before it, one where the persistent workgroups get unequal tile counts)."""
     a, w, alpha, beta = problem(51 + T, T, K, N, full_range=True)
     got = run_gpu(a, w, None, None, capi.LINEAR_RAW_INT32, a_il=True, w_il=True)
     ref = oracle.int8_linear(a, w, epilogue=oracle.LINEAR_RAW_INT32)
