@@ -592,10 +592,6 @@ int launch_interleaved(hipStream_t stream, int32_t total, int8_t const* in, int8
 {
     dim3 const grid((unsigned) ceil_div(total, TOK));
     dim3 const block(W * kWaveSize);
-    static int const dynLds = [] {
-        char const* e = getenv("TRTAMD_SKIPLN_LDS");
-        return e ? atoi(e) : 0;
-    }();
     if (preln)
     {
         hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, true>), grid, block, 0, stream, total, in, skip, beta,
@@ -603,7 +599,7 @@ int launch_interleaved(hipStream_t stream, int32_t total, int8_t const* in, int8
     }
     else
     {
-        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, false>), grid, block, dynLds, stream, total, in, skip, beta,
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, false>), grid, block, 0, stream, total, in, skip, beta,
             gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
     }
     return check_launch("skipln_interleaved_kernel");
@@ -640,28 +636,16 @@ int skipln_interleaved(hipStream_t stream, bool large, bool mtron, int32_t ld, i
     float const eps = large ? 1.1920928955078125e-07f : 0.0009765625f;
     float const pmin = large ? -128.f : -127.f;
     int8_t* pre = mtron ? preln : nullptr;
-    // wavefronts per 8-token group: enough that every lane keeps at most 8 x 16 bytes per tensor, and
-    // small work units so that the loads of one workgroup overlap the arithmetic of another
-    static int const tune = [] {
-        char const* e = getenv("TRTAMD_SKIPLN_W");
-        return e ? atoi(e) : 0;
-    }();
+    // 32 tokens per workgroup and enough wavefronts that a lane keeps at most 8 x 16 bytes per tensor; other
+    // splits (8 or 16 tokens, 2 to 16 wavefronts) measured the same or slower at 4 k to 33 k tokens
 #define TRTAMD_IL(G, W, TOK)                                                                                          \
     return launch_interleaved<G, W, TOK>(stream, total, in, skip, beta, gamma, out, pre, dqIn, dqSkip, qScale,         \
         qSkipScale, eps, pmin)
     switch (ld)
     {
     case 768:
-        if (tune == 1) { TRTAMD_IL(24, 3, 8); }
-        if (tune == 2) { TRTAMD_IL(24, 3, 16); }
-        if (tune == 3) { TRTAMD_IL(24, 3, 32); }
         TRTAMD_IL(24, 6, 32);
     case 1024:
-        if (tune == 1) { TRTAMD_IL(32, 2, 8); }
-        if (tune == 2) { TRTAMD_IL(32, 4, 16); }
-        if (tune == 3) { TRTAMD_IL(32, 4, 32); }
-        if (tune == 4) { TRTAMD_IL(32, 2, 16); }
-        if (tune == 5) { TRTAMD_IL(32, 16, 32); }
         TRTAMD_IL(32, 8, 32);
     case 1536: TRTAMD_IL(48, 8, 32);
     case 2048: TRTAMD_IL(64, 8, 32);
