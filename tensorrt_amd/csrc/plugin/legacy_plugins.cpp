@@ -128,6 +128,10 @@ void parseStream(void const* data, size_t length, ParsedStream& ps)
         throw std::runtime_error("not a plugin stream written by this library");
     }
     uint32_t const n = get32();
+    if (static_cast<size_t>(n) > length / 16)
+    {
+        throw std::runtime_error("serialised plugin is truncated"); // every field takes at least its 16-byte header
+    }
     ps.names.reserve(n);
     for (uint32_t i = 0; i < n; ++i)
     {
@@ -342,8 +346,8 @@ private:
 };
 
 // How many inputs each operator takes, from its serialised configuration (needed because the V2
-// enqueue() does not say): SkipLayerNorm 2; EmbLayerNorm fixed 3, var-seqlen 4; QKV-to-context 1 + mask
-// (fixed), 4 (var-seqlen), 3 (interleaved).
+// enqueue() does not say): SkipLayerNorm 2; EmbLayerNorm fixed 3, var-seqlen 4; QKV-to-context 1 + has_mask
+// + 2 * var_seqlen, interleaved 3.
 int32_t inputsOf(char const* pluginName, char const* legacyVersion, IPluginV3* p)
 {
     std::string const name = pluginName;
@@ -360,20 +364,22 @@ int32_t inputsOf(char const* pluginName, char const* legacyVersion, IPluginV3* p
     {
         return 3;
     }
-    if (v == 2)
-    {
-        return 4;
-    }
-    // fixed-length attention: the mask input exists when has_mask was set
     PluginFieldCollection const* fc = cap<IPluginV3OneRuntime>(p, PluginCapabilityType::kRUNTIME)->getFieldsToSerialize();
-    for (int32_t i = 0; fc && i < fc->nbFields; ++i)
-    {
-        if (std::strcmp(fc->fields[i].name, "has_mask") == 0 && fc->fields[i].data)
+    auto flag = [&](char const* field, int32_t fallback) {
+        for (int32_t i = 0; fc && i < fc->nbFields; ++i)
         {
-            return 1 + (*static_cast<int32_t const*>(fc->fields[i].data) != 0 ? 1 : 0);
+            if (std::strcmp(fc->fields[i].name, field) == 0 && fc->fields[i].data
+                && fc->fields[i].type == PluginFieldType::kINT32 && fc->fields[i].length >= 1)
+            {
+                return *static_cast<int32_t const*>(fc->fields[i].data);
+            }
         }
-    }
-    return 2;
+        return fallback;
+    };
+    // qkv, the mask when has_mask was set, and for version 2 cu_seqlens and the max-length dummy when var_seqlen is
+    // set (plugin/bertQKVToContextPlugin/qkvToContextPluginLegacy.cpp, QKVToContextVarSeqlenPluginDynamicLegacy)
+    int32_t const varSeqlen = v == 2 && flag("var_seqlen", 0) != 0 ? 1 : 0;
+    return 1 + (flag("has_mask", 1) != 0 ? 1 : 0) + 2 * varSeqlen;
 }
 
 class LegacyCreator : public IPluginCreator
@@ -415,6 +421,10 @@ public:
         catch (std::exception const& e)
         {
             logError(e.what());
+        }
+        catch (...)
+        {
+            logError("unknown error while reading the serialised plugin");
         }
         return nullptr;
     }

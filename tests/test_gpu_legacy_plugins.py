@@ -221,3 +221,27 @@ def test_legacy_qkv_varseqlen(reg, legacy, current, dt):
         s2 = np.float32(np.float32(dqp * s_q) / s_ctx)
         ref = oracle.mha_fused_i8_packed(q, cu, N, d, s1, np.float32(1) / dqp, s2)
         assert_int8_close(oracle.deinterleave(out, T, hidden), ref, what="legacy QKV v3", max_frac_off=0.002)
+
+
+@pytest.mark.parametrize("has_mask", [0, 1])
+def test_legacy_qkv_version_2_without_var_seqlen(reg, has_mask):
+    """Version 2 with var_seqlen = 0 is the fixed-length operator: qkv and, with has_mask, the mask.  The
+    deserialised plugin must know its input count from the stream alone (enqueue does not state it)."""
+    r = rng(36 + has_mask)
+    S, B, N, d = 40, 3, 2, 32
+    hidden = N * d
+    qkv = (r.standard_normal((S, B, 3 * hidden)) / 4).astype(np.float32)
+    lens = r.integers(1, S + 1, B).astype(np.int32)
+    fs = [i32("type_id", 0), i32("hidden_size", hidden), i32("num_heads", N), i32("has_mask", has_mask),
+          i32("var_seqlen", 0)]
+    ins = [TensorDesc([S, B, 3 * hidden, 1, 1], DataType.FLOAT)]
+    inputs = [dev(qkv)]
+    if has_mask:
+        ins.append(TensorDesc([B], DataType.INT32))
+        inputs.append(dev(lens))
+    outs = [TensorDesc([S, B, hidden, 1, 1], DataType.FLOAT)]
+    lp, cp = both(reg, QKV, "2", "5", fs, ins, outs)
+    ws_bytes = cp.get_workspace_size(ins, outs)
+    (out,) = run_both(lp, cp, ins, outs, inputs, [(S, B, hidden)], [np.float32], ws_bytes)
+    ref = oracle.mha_unfused_fixed(qkv, S, B, N, d, lens if has_mask else None)
+    assert_fp_close(out, ref, what="legacy QKV v2, fixed length")
