@@ -129,14 +129,14 @@ __device__ inline int frag_offset(int row, int half)
 // of four consecutive channels.  For the INT8 outputs the two lanes that share a token trade two packed dwords
 // (v_permlane32_swap), after which lane l holds the 16 consecutive channels 16*(l/32)..+15 and stores them with
 // one 16-byte write.
-template <bool IL_OUT, int EPI>
+template <bool IL_OUT, int EPI, bool FULL = false>
 __device__ __forceinline__ void store_block(
     LinearArgs const& p, AccT<EPI> const& acc, int const c0, int const tb, float const* sAlpha, float const* sBeta)
 {
     int const lane = threadIdx.x & 63;
     int const hi = lane >> 5;
     int const t = tb + (lane & 31);
-    bool const live = t < p.T;
+    bool const live = FULL || t < p.T; // FULL: the block lies inside the problem and is stored unconditionally
     f32x4 al[4], be[4];
     if constexpr (EPI != kRAW)
     {
@@ -636,6 +636,235 @@ __device__ __forceinline__ void linear_tile_run(
     }
 }
 
+// 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane i's bytes land at LDS byte
+// address ldsAddr + 16 i, so one instruction of a wavefront fills 1 KB; ldsAddr is wave-uniform and travels in M0.
+// The data never passes through vector registers, and completion is counted by vmcnt like any vector-memory load.
+// Written as inline assembly on purpose: the compiler then neither counts these loads nor orders LDS reads behind
+// them, and the kernel below places its own s_waitcnt where a stage must have landed.
+__device__ __forceinline__ void load_to_lds16(void const* g, uint32_t ldsAddr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(ldsAddr) : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(N) alone (the other counters at their maxima): gfx9 encoding, vmcnt in bits 3:0 and 15:14
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// The persistent run of 256 x 256 tiles with the stages brought in by direct-to-LDS loads: a ring of four LDS stage
+// buffers, stage k+3 requested while stage k is multiplied, no staging registers, no LDS-write instructions and
+// nothing for a wavefront to wait for before the barrier except loads issued two steps earlier.  Both operands in
+// the 32-interleaved layout (a fragment is then 1 KB of contiguous memory, which one instruction moves; the LDS
+// swizzle is applied on the source side: lane i fetches the 16 bytes that belong at LDS offset 16 i), INT8 output,
+// N a multiple of 256 and K of 256 (the ring index is then the stage index modulo 4 in every tile).
+template <bool IL_OUT, int EPI, typename Origin>
+__device__ __forceinline__ void linear_tile_run_dma(
+    LinearArgs const& p, int const count, Origin origin, uint8_t* __restrict__ lds, float* sScale)
+{
+    constexpr int WM = 2, WN = 4, MT = 4, NT = 2, NWAVES = 8;
+    constexpr int AF = (kBigTile / 32) * 2;
+    constexpr int BF = (kBigTile / 32) * 2;
+    constexpr int LA = AF / NWAVES;
+    constexpr int LB = BF / NWAVES;
+    constexpr int STAGE = (AF + BF) * 1024;
+    constexpr int kLoads = LA + LB;           // direct loads per wavefront and stage
+    constexpr int kStores = MT * NT;          // global stores per wavefront in a tile's epilogue
+    static_assert(EPI == kAFFINE || EPI == kGELU, "one 16-byte store per accumulator block");
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const wm = wave / WN;
+    int const wn = wave % WN;
+    uint32_t const ldsBase = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lds;
+    uint32_t const scaleBase = (uint32_t) (size_t) (__attribute__((address_space(3))) float*) sScale;
+
+    // lane i of a unit's load supplies LDS offset 16 i of the fragment: row i/2, and the half that the swizzle puts there
+    int const r = lane >> 1;
+    uint32_t const half = (uint32_t) ((lane & 1) ^ ((r >> 3) & 1));
+    auto address = [&](int n0, int t0, uint32_t(&oa)[LA], uint32_t(&ob)[LB]) {
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            int const u = q * NWAVES + wave, rb = u >> 1, sel = u & 1;
+            oa[q] = ((uint32_t) sel * (uint32_t) p.N + (uint32_t) (n0 + rb * 32 + r)) * 32u + half * 16u;
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            int const u = q * NWAVES + wave, rb = u >> 1, sel = u & 1;
+            ob[q] = ((uint32_t) sel * (uint32_t) p.T + (uint32_t) (t0 + rb * 32 + r)) * 32u + half * 16u;
+        }
+    };
+    uint32_t const stepA = 2u * (uint32_t) p.N * 32u;
+    uint32_t const stepB = 2u * (uint32_t) p.T * 32u;
+    int const nk = p.K / 64; // a multiple of 4
+
+    uint32_t oaC[LA], obC[LB], oaN[LA], obN[LB];
+    // stage kt of the current tile (or stage kt - nk of the next one) into ring slot `slot`
+    auto fetch = [&](int kt, int slot) {
+        bool const next = kt >= nk;
+        uint32_t const k = (uint32_t) (next ? kt - nk : kt);
+        uint32_t const dst = ldsBase + (uint32_t) slot * STAGE;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            load_to_lds16(p.w + (next ? oaN[q] : oaC[q]) + k * stepA, dst + (uint32_t) (q * NWAVES + wave) * 1024u);
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            load_to_lds16(p.a + (next ? obN[q] : obC[q]) + k * stepB, dst + (uint32_t) (AF + q * NWAVES + wave) * 1024u);
+        }
+    };
+
+    AccT<EPI> acc[MT][NT];
+    int const readOff = frag_offset(lane & 31, lane >> 5);
+    auto multiply = [&](int slot) {
+        uint8_t const* base = lds + slot * STAGE + readOff;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+        {
+            i32x4 fa[MT], fb[NT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+            {
+                fa[i] = *reinterpret_cast<i32x4 const*>(base + ((wm * MT + i) * 2 + ks) * 1024);
+            }
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+            {
+                fb[j] = *reinterpret_cast<i32x4 const*>(base + (AF + (wn * NT + j) * 2 + ks) * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+            {
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                {
+                    acc[i][j] = mma<EPI>(fa[i], fb[j], acc[i][j]);
+                }
+            }
+        }
+    };
+    // scale / offset vectors of a tile, 256 binary32 values each: one direct load by wave 0 and one by wave 1
+    auto fetch_scales = [&](int n0, int parity) {
+        if (wave < 2)
+        {
+            float const* src = (wave == 0 ? p.alpha : p.beta) + n0 + lane * 4;
+            load_to_lds16(src, scaleBase + (uint32_t) ((parity * 2 + wave) * kBigTile) * 4u);
+        }
+    };
+    auto scales = [&](int parity, int which) { return sScale + (parity * 2 + which) * kBigTile; };
+    // one step: request stage k+3, multiply stage k, make sure this wavefront's part of stage k+1 has landed, meet
+    // the others.  vmcnt counts the kLoads of stages k+2 and k+3 behind it, and `extra` operations known to sit
+    // between (epilogue stores), which must not be waited for.
+    auto step = [&](int k, auto slotTag, auto extraTag) {
+        constexpr int SLOT = decltype(slotTag)::value;
+        constexpr int EXTRA = decltype(extraTag)::value;
+        fetch(k + 3, (SLOT + 3) & 3);
+        multiply(SLOT);
+        wait_vmcnt<2 * kLoads + EXTRA>();
+        __syncthreads();
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+    using NoExtra = std::integral_constant<int, 0>;
+    using Stores = std::integral_constant<int, kStores>;
+
+    int n0, t0;
+    origin(0, n0, t0);
+    address(n0, t0, oaC, obC);
+#pragma unroll
+    for (int q = 0; q < LA; ++q)
+    {
+        oaN[q] = oaC[q];
+    }
+#pragma unroll
+    for (int q = 0; q < LB; ++q)
+    {
+        obN[q] = obC[q];
+    }
+    fetch_scales(n0, 0);
+    fetch(0, 0);
+    fetch(1, 1);
+    fetch(2, 2);
+    wait_vmcnt<2 * kLoads>();
+    __syncthreads();
+    for (int j = 0; j < count; ++j)
+    {
+        int n1 = n0, t1 = t0;
+        if (j + 1 < count)
+        {
+            origin(j + 1, n1, t1);
+        }
+        address(n1, t1, oaN, obN);
+        fetch_scales(n1, (j + 1) & 1);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+        {
+#pragma unroll
+            for (int jj = 0; jj < NT; ++jj)
+            {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                {
+                    acc[i][jj][v] = 0;
+                }
+            }
+        }
+        // the first two steps after an epilogue have its stores between the stage they wait for and the newer loads
+        if (j == 0)
+        {
+            step(0, S0{}, NoExtra{});
+            step(1, S1{}, NoExtra{});
+        }
+        else
+        {
+            step(0, S0{}, Stores{});
+            step(1, S1{}, Stores{});
+        }
+        step(2, S2{}, NoExtra{});
+        step(3, S3{}, NoExtra{});
+        for (int k = 4; k < nk; k += 4)
+        {
+            step(k, S0{}, NoExtra{});
+            step(k + 1, S1{}, NoExtra{});
+            step(k + 2, S2{}, NoExtra{});
+            step(k + 3, S3{}, NoExtra{});
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+        {
+#pragma unroll
+            for (int jj = 0; jj < NT; ++jj)
+            {
+                int const cl = (wm * MT + i) * 32;
+                store_block<IL_OUT, EPI, true>(p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, scales(j & 1, 0) + cl,
+                    scales(j & 1, 1) + cl);
+            }
+        }
+        n0 = n1;
+        t0 = t1;
+#pragma unroll
+        for (int q = 0; q < LA; ++q)
+        {
+            oaC[q] = oaN[q];
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+        {
+            obC[q] = obN[q];
+        }
+    }
+    // the loads requested for a tile after the last one are still in flight: they must land before the LDS is released
+    wait_vmcnt<0>();
+}
+
 // Tokens [0, 256*tokMain) are cut into 256 x 256 tiles (workgroups 0 .. mainTiles-1); what is left, which
 // would otherwise be a last round of big tiles on a fraction of the CUs, is cut into 128 x 128 tiles that
 // spread over all of them.
@@ -702,6 +931,37 @@ __global__ __launch_bounds__(512) void int8_linear_persistent_kernel(LinearArgs 
     }
 }
 
+// The persistent tile plan with direct-to-LDS loads for the 256 x 256 tiles.
+template <bool IL_OUT, int EPI>
+__global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[4 * 2 * (kBig / 32) * 2 * 1024];
+    __shared__ __attribute__((aligned(16))) float sScale[2 * 2 * kBig];
+    if ((int) blockIdx.x < p.persist)
+    {
+        uint32_t const pw = (uint32_t) p.panel;
+        uint32_t const perPanel = (uint32_t) p.tokMain * pw;
+        int const count = (p.mainTiles - (int) blockIdx.x + p.persist - 1) / p.persist;
+        auto origin = [&](int j, int& n0, int& t0) {
+            uint32_t const tile = xcd_remap(blockIdx.x + (uint32_t) j * (uint32_t) p.persist, (uint32_t) p.mainTiles);
+            uint32_t const pan = tile / perPanel, rem = tile % perPanel;
+            n0 = (int) (pan * pw + rem % pw) * kBig;
+            t0 = (int) (rem / pw) * kBig;
+        };
+        linear_tile_run_dma<IL_OUT, EPI>(p, count, origin, lds, sScale);
+    }
+    else
+    {
+        uint32_t const nbm = (uint32_t) ((p.N + kSmall - 1) / kSmall);
+        uint32_t const tile = blockIdx.x - (uint32_t) p.persist;
+        auto origin = [&](int, int& n0, int& t0) {
+            n0 = (int) (tile % nbm) * kSmall;
+            t0 = p.tokMain * kBig + (int) (tile / nbm) * kSmall;
+        };
+        linear_tile_run<2, 4, 2, 1, true, true, IL_OUT, EPI>(p, 1, origin, lds, sScale);
+    }
+}
+
 int num_cus()
 {
     static int const n = [] {
@@ -759,6 +1019,18 @@ int launch_shape(hipStream_t stream, LinearArgs a)
     {
         a.persist = a.mainTiles < cus ? a.mainTiles : cus;
         int64_t const pgrid = grid - a.mainTiles + a.persist;
+        static int const direct = [] {
+            char const* e = getenv("TRTAMD_LINEAR_DIRECT");
+            return e ? atoi(e) : 0;
+        }();
+        if constexpr (IL_W && IL_IN && (EPI == kAFFINE || EPI == kGELU))
+        {
+            if (direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
+            {
+                hipLaunchKernelGGL((int8_linear_dma_kernel<IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0, stream, a);
+                return check_launch("int8_linear_dma_kernel");
+            }
+        }
         hipLaunchKernelGGL((int8_linear_persistent_kernel<IL_W, IL_IN, IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0,
             stream, a);
         return check_launch("int8_linear_persistent_kernel");

@@ -114,7 +114,7 @@ def test_affine_fp16(T, K, N):
 
 
 @pytest.mark.parametrize("T,K,N", [(8229, 128, 3072), (16500, 64, 1024), (70000, 64, 256), (9600, 128, 1024),
-                                   (28165, 128, 1024)])
+                                   (28165, 128, 1024), (9600, 256, 1024), (28165, 512, 1024), (20000, 1024, 512)])
 def test_large_problems_mix_both_tile_sizes(T, K, N):
     """Enough 256 x 256 tiles for whole rounds of the chip, plus a remainder in 128 x 128 tiles.  The last two
     sizes leave more than half a round of large tiles, which then runs as a partial round (one with no whole
@@ -129,6 +129,12 @@ def test_large_problems_mix_both_tile_sizes(T, K, N):
     got_lin = run_gpu(a, w, alpha, beta, capi.LINEAR_GELU, out_scale=0.5)
     ref_lin = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_GELU, out_scale=0.5)
     assert_int8_close(got_lin, ref_lin, what="gelu, linear layouts", max_frac_off=2e-3)
+    got_il = run_gpu(a, w, alpha, beta, capi.LINEAR_GELU, out_scale=0.5, a_il=True, w_il=True, out_il=True)
+    ref_il = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_GELU, out_scale=0.5, out_interleaved=True)
+    assert_int8_close(got_il, ref_il, what="gelu, interleaved layouts", max_frac_off=2e-3)
+    got_mixed = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=True, w_il=True, out_il=False)
+    ref_mixed = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE)
+    assert_int8_close(got_mixed, ref_mixed, what="affine, interleaved operands, linear output", max_frac_off=1e-3)
 
 
 def test_output_untouched_beyond_the_problem():
