@@ -641,10 +641,13 @@ __device__ __forceinline__ void linear_tile_run(
 // The data never passes through vector registers, and completion is counted by vmcnt like any vector-memory load.
 // Written as inline assembly on purpose: the compiler then neither counts these loads nor orders LDS reads behind
 // them, and the kernel below places its own s_waitcnt where a stage must have landed.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm" // M0 is named as clobbered on purpose
 __device__ __forceinline__ void load_to_lds16(void const* g, uint32_t ldsAddr)
 {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(ldsAddr) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // s_waitcnt vmcnt(N) alone (the other counters at their maxima): gfx9 encoding, vmcnt in bits 3:0 and 15:14
 template <int N>
@@ -664,7 +667,7 @@ template <bool IL_OUT, int EPI, typename Origin>
 __device__ __forceinline__ void linear_tile_run_dma(
     LinearArgs const& p, int const count, Origin origin, uint8_t* __restrict__ lds, float* sScale)
 {
-    constexpr int WM = 2, WN = 4, MT = 4, NT = 2, NWAVES = 8;
+    constexpr int WN = 4, MT = 4, NT = 2, NWAVES = 8;
     constexpr int AF = (kBigTile / 32) * 2;
     constexpr int BF = (kBigTile / 32) * 2;
     constexpr int LA = AF / NWAVES;
@@ -803,7 +806,6 @@ __device__ __forceinline__ void linear_tile_run_dma(
             origin(j + 1, n1, t1);
         }
         address(n1, t1, oaN, obN);
-        fetch_scales(n1, (j + 1) & 1);
 #pragma unroll
         for (int i = 0; i < MT; ++i)
         {
@@ -817,15 +819,20 @@ __device__ __forceinline__ void linear_tile_run_dma(
                 }
             }
         }
-        // the first two steps after an epilogue have its stores between the stage they wait for and the newer loads
+        // The first two steps after an epilogue have its stores between the stage they wait for and the newer loads.
+        // The next tile's scale vectors go into the buffer the previous tile's epilogue read: only after the first
+        // barrier of this tile has every wavefront left that epilogue.  (On the two wavefronts that fetch them the
+        // waits below then count one operation too few, which only makes them wait for one more load.)
         if (j == 0)
         {
             step(0, S0{}, NoExtra{});
+            fetch_scales(n1, (j + 1) & 1);
             step(1, S1{}, NoExtra{});
         }
         else
         {
             step(0, S0{}, Stores{});
+            fetch_scales(n1, (j + 1) & 1);
             step(1, S1{}, Stores{});
         }
         step(2, S2{}, NoExtra{});
@@ -1021,7 +1028,7 @@ int launch_shape(hipStream_t stream, LinearArgs a)
         int64_t const pgrid = grid - a.mainTiles + a.persist;
         static int const direct = [] {
             char const* e = getenv("TRTAMD_LINEAR_DIRECT");
-            return e ? atoi(e) : 0;
+            return e ? atoi(e) : 1;
         }();
         if constexpr (IL_W && IL_IN && (EPI == kAFFINE || EPI == kGELU))
         {

@@ -160,3 +160,47 @@ def test_int8_skip_layer_norm_at_benchmark_size(api):
     order = r.permutation(total)
     moved, _, _ = run(x[order], s[order])
     assert np.array_equal(oracle.deinterleave(moved, total, ld), oracle.deinterleave(got, total, ld)[order])
+
+
+@pytest.mark.parametrize("K,N,gelu", [(1024, 4096, True), (4096, 1024, False), (1024, 3072, False)])
+def test_int8_linear_at_benchmark_size(K, N, gelu):
+    """The encoder's linear layers at 33289 tokens: every output row depends on its own input row only, so the
+    oracle is run on a sample of rows (the first and last ones, rows either side of every 256-token tile edge of one
+    region, and random ones) and must match there; a second launch on a row permutation must give the permuted
+    output everywhere."""
+    import torch
+    from tensorrt_amd import capi
+    r = rng(5)
+    T = 33289
+    a = np.clip(np.rint(r.standard_normal((T, K)) * 30), -127, 127).astype(np.int8)
+    w = np.clip(np.rint(r.standard_normal((N, K)) * 30), -127, 127).astype(np.int8)
+    alpha = (r.uniform(0.5, 1.5, N) * (3.0 / (30 * 30 * np.sqrt(K)))).astype(np.float32)
+    beta = (0.3 * r.standard_normal(N)).astype(np.float32)
+    if not gelu:
+        alpha, beta = alpha * np.float32(30), beta * np.float32(30)   # outputs spread over the INT8 range
+    api = capi.api()
+    dw = dev(oracle.interleave(w).reshape(K // 32, N, 32))
+    dal, dbe = dev(alpha), dev(beta)
+
+    def run(x):
+        da = dev(oracle.interleave(x).reshape(K // 32, T, 32))
+        out = dev_empty((N // 32, T, 32), np.int8, fill=0)
+        p = capi.Int8LinearParams()
+        p.a, p.w, p.alpha, p.beta, p.out = da.data_ptr(), dw.data_ptr(), dal.data_ptr(), dbe.data_ptr(), out.data_ptr()
+        p.T, p.K, p.N = T, K, N
+        p.a_interleaved = p.w_interleaved = p.out_interleaved = 1
+        p.epilogue, p.out_scale = (capi.LINEAR_GELU if gelu else capi.LINEAR_AFFINE), 30.0
+        api.check(api.int8_linear(torch.cuda.current_stream().cuda_stream, C.byref(p)))
+        torch.cuda.synchronize()
+        return oracle.deinterleave(host(out).ravel(), T, N)
+
+    got = run(a)
+    edges = np.concatenate([np.arange(e - 2, e + 2) for e in range(256, 256 * 12, 256)])
+    rows = np.unique(np.concatenate([np.arange(4), np.arange(T - 4, T), edges, np.arange(32768 - 3, 32768 + 3),
+                                     r.integers(0, T, 1200)]))
+    ref = oracle.int8_linear(a[rows], w, alpha, beta, oracle.LINEAR_GELU if gelu else oracle.LINEAR_AFFINE,
+                             out_scale=30.0)
+    assert np.abs(ref.astype(np.int32)).max() > 60
+    assert_int8_close(got[rows], ref, what="sampled rows vs oracle", max_frac_off=2e-3)
+    order = r.permutation(T)
+    assert np.array_equal(run(a[order]), got[order])

@@ -114,7 +114,7 @@ def test_affine_fp16(T, K, N):
 
 
 @pytest.mark.parametrize("T,K,N", [(8229, 128, 3072), (16500, 64, 1024), (70000, 64, 256), (9600, 128, 1024),
-                                   (28165, 128, 1024), (9600, 256, 1024), (28165, 512, 1024), (20000, 1024, 512)])
+                                   (28165, 128, 1024), (9600, 256, 1024), (28165, 512, 1024), (20000, 1024, 512), (70000, 256, 1024)])
 def test_large_problems_mix_both_tile_sizes(T, K, N):
     """Enough 256 x 256 tiles for whole rounds of the chip, plus a remainder in 128 x 128 tiles.  The last two
     sizes leave more than half a round of large tiles, which then runs as a partial round (one with no whole
