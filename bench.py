@@ -224,7 +224,7 @@ def run_encoder(args, api, torch):
                       + (", replayed from a captured graph" if args.graph else ""),
         },
         "roofline": {
-            "kernel": "int8_linear_persistent_kernel<true,true,true,GELU> (feed-forward 1)",
+            "kernel": "int8_linear_dma_kernel<true,GELU> (feed-forward 1)",
             "bound": "mfma",
             "achieved": table[dom]["TOP/s"],
             "peak": PEAK_INT8_OPS / 1e12,
