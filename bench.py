@@ -269,6 +269,56 @@ def run_encoder(args, api, torch):
     return out
 
 
+def run_encoder_fp16(args, torch):
+    """The same 24-layer BERT-large network in FP16 (not the contract's metric: an extra workload that times the FP16
+    half of the plugin family in place: EmbLayerNorm v4, fused FP16 attention v5, SkipLayerNorm v6, FP16 linear layers)."""
+    from tensorrt_amd.encoder import EncoderConfig
+    from tensorrt_amd.encoder_fp16 import Fp16BertEncoder
+    cfg = EncoderConfig(layers=args.layers, seed=args.seed, max_seqlen=args.seqlen)
+    r = np.random.default_rng(args.seed)
+    lens = r.integers(128, args.seqlen + 1, args.batch)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    ids = r.integers(0, cfg.vocab, T).astype(np.int32)
+    segs = r.integers(0, 2, T).astype(np.int32)
+    enc = Fp16BertEncoder(cfg)
+    out = enc.enqueue(ids, segs, cu)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out.float()).all())
+    clock_ramp(torch, enc.enqueue)
+    for _ in range(max(args.warmup, 1)):
+        enc.enqueue()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        enc.enqueue()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    flops = enc.flops()
+    return {
+        "metric": "BERT-large FP16 S=384 seq/s on 1 GPU (extra workload)",
+        "value": round(args.batch / (ms_step * 1e-3), 1),
+        "unit": "sequences/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16",
+        "data": "synthetic",
+        "config": {"workload": f"full {cfg.layers}-layer BERT-large FP16 encoder: EmbLayerNorm v4, per layer FP16 GEMM / "
+                               "QKV-to-context v5 (fused FP16, cu_seqlens) / FP16 GEMM / SkipLayerNorm v6 / FP16 GEMM+GELU / "
+                               "FP16 GEMM / SkipLayerNorm v6; random-init weights",
+                   "batch": args.batch, "max_seqlen": args.seqlen, "heads": cfg.heads, "hidden": cfg.hidden,
+                   "ffn": cfg.ffn, "layers": cfg.layers, "tokens": T, "runner": "python"},
+        "roofline": {"kernel": "whole pass (linear layers + attention)", "bound": "mfma",
+                     "achieved": round(flops / (ms_step * 1e-3) / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": round(flops / (ms_step * 1e-3) / 2.5e15, 4), "traffic": None},
+    }
+
+
 def cpu_baseline_torch(enc, cu, lens, torch, budget_s=8.0):
     """What a CPU inference library does with the same network: the de-quantised FP32 subgraph of one layer
     (MatMul + bias, per-sequence softmax attention, Add + LayerNormalization, erf GELU) through torch's CPU
@@ -374,7 +424,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", choices=["encoder", "layer"], default="encoder")
+    ap.add_argument("--workload", choices=["encoder", "layer", "encoder-fp16"], default="encoder")
     ap.add_argument("--layers", type=int, default=24, help="encoder workload only")
     ap.add_argument("--graph", action="store_true",
                     help="encoder workload: record the native runner's pass into a graph and time its replays")
@@ -399,6 +449,12 @@ def main():
         sys.exit(1)
     from tensorrt_amd import capi
     api = capi.api()   # raises if the HIP library is missing: there is no fallback
+    if args.workload == "encoder-fp16":
+        args.batch = args.batch or 128
+        if args.steps == 1000 and args.warmup == 200:
+            args.steps, args.warmup = 10, 3
+        print(json.dumps(run_encoder_fp16(args, torch)))
+        return
     if args.workload == "encoder":
         args.batch = args.batch or 128
         if args.steps == 1000 and args.warmup == 200:   # the layer workload's defaults: a pass is ~300x longer
