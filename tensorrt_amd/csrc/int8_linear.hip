@@ -659,11 +659,16 @@ __device__ __forceinline__ void wait_vmcnt()
 
 // The persistent run of 256 x 256 tiles with the stages brought in by direct-to-LDS loads: a ring of four LDS stage
 // buffers, stage k+3 requested while stage k is multiplied, no staging registers, no LDS-write instructions and
-// nothing for a wavefront to wait for before the barrier except loads issued two steps earlier.  Both operands in
-// the 32-interleaved layout (a fragment is then 1 KB of contiguous memory, which one instruction moves; the LDS
-// swizzle is applied on the source side: lane i fetches the 16 bytes that belong at LDS offset 16 i), INT8 output,
-// N a multiple of 256 and K of 256 (the ring index is then the stage index modulo 4 in every tile).
-template <bool IL_OUT, int EPI, typename Origin>
+// nothing for a wavefront to wait for before the barrier except loads issued two steps earlier.  N a multiple of 256
+// and K of 256 bytes (the ring index is then the stage index modulo 4 in every tile).  One instruction fills 1 KB of
+// LDS with lane i's 16 bytes at offset 16 i, so the LDS swizzle is applied on the source side: lane i fetches the
+// 16 bytes that belong there.
+//   IL (both operands 32-interleaved): a load unit is one fragment, 32 rows x 32 bytes, contiguous in memory.
+//   otherwise (both operands linear [R][K], also the FP16 layers): a load unit is 16 rows x 64 bytes (four lanes
+//   per row, 64 contiguous bytes of it); in LDS the 16-byte chunk c of row r sits at chunk c ^ (r / 4), which makes
+//   the fragment reads (16 rows x one chunk per 16 lanes) conflict-free; fragment (block, ks) takes chunks 2 ks and
+//   2 ks + 1 of the block's two units.
+template <bool IL, bool IL_OUT, int EPI, typename Origin>
 __device__ __forceinline__ void linear_tile_run_dma(
     LinearArgs const& p, int const count, Origin origin, uint8_t* __restrict__ lds, float* sScale)
 {
@@ -674,8 +679,9 @@ __device__ __forceinline__ void linear_tile_run_dma(
     constexpr int LB = BF / NWAVES;
     constexpr int STAGE = (AF + BF) * 1024;
     constexpr int kLoads = LA + LB;           // direct loads per wavefront and stage
-    constexpr int kStores = MT * NT;          // global stores per wavefront in a tile's epilogue
-    static_assert(EPI == kAFFINE || EPI == kGELU, "one 16-byte store per accumulator block");
+    // global stores per wavefront in a tile's epilogue: one 16-byte store per accumulator block (INT8), four of 8 bytes (FP16)
+    constexpr int kStores = MT * NT * (EPI >= kF16_AFFINE ? 4 : 1);
+    static_assert(EPI == kAFFINE || EPI == kGELU || EPI == kF16_AFFINE || EPI == kF16_GELU, "store count per block");
 
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -684,25 +690,36 @@ __device__ __forceinline__ void linear_tile_run_dma(
     uint32_t const ldsBase = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lds;
     uint32_t const scaleBase = (uint32_t) (size_t) (__attribute__((address_space(3))) float*) sScale;
 
-    // lane i of a unit's load supplies LDS offset 16 i of the fragment: row i/2, and the half that the swizzle puts there
-    int const r = lane >> 1;
-    uint32_t const half = (uint32_t) ((lane & 1) ^ ((r >> 3) & 1));
+    // lane i of a unit's load supplies LDS offset 16 i of the unit
+    auto unit_offset = [&](int u, int row0, int R) -> uint32_t {
+        int const rb = u >> 1, sel = u & 1;
+        if constexpr (IL)
+        {
+            int const r = lane >> 1; // row of the fragment; the half that the swizzle puts at this offset
+            uint32_t const half = (uint32_t) ((lane & 1) ^ ((r >> 3) & 1));
+            return ((uint32_t) sel * (uint32_t) R + (uint32_t) (row0 + rb * 32 + r)) * 32u + half * 16u;
+        }
+        else
+        {
+            int const rr = lane >> 2; // row of the 16-row unit; the chunk that the swizzle puts at this offset
+            uint32_t const chunk = (uint32_t) ((lane & 3) ^ (rr >> 2));
+            return (uint32_t) (row0 + rb * 32 + sel * 16 + rr) * (uint32_t) p.K + chunk * 16u;
+        }
+    };
     auto address = [&](int n0, int t0, uint32_t(&oa)[LA], uint32_t(&ob)[LB]) {
 #pragma unroll
         for (int q = 0; q < LA; ++q)
         {
-            int const u = q * NWAVES + wave, rb = u >> 1, sel = u & 1;
-            oa[q] = ((uint32_t) sel * (uint32_t) p.N + (uint32_t) (n0 + rb * 32 + r)) * 32u + half * 16u;
+            oa[q] = unit_offset(q * NWAVES + wave, n0, p.N);
         }
 #pragma unroll
         for (int q = 0; q < LB; ++q)
         {
-            int const u = q * NWAVES + wave, rb = u >> 1, sel = u & 1;
-            ob[q] = ((uint32_t) sel * (uint32_t) p.T + (uint32_t) (t0 + rb * 32 + r)) * 32u + half * 16u;
+            ob[q] = unit_offset(q * NWAVES + wave, t0, p.T);
         }
     };
-    uint32_t const stepA = 2u * (uint32_t) p.N * 32u;
-    uint32_t const stepB = 2u * (uint32_t) p.T * 32u;
+    uint32_t const stepA = IL ? 2u * (uint32_t) p.N * 32u : 64u;
+    uint32_t const stepB = IL ? 2u * (uint32_t) p.T * 32u : 64u;
     int const nk = p.K / 64; // a multiple of 4
 
     uint32_t oaC[LA], obC[LB], oaN[LA], obN[LB];
@@ -724,9 +741,23 @@ __device__ __forceinline__ void linear_tile_run_dma(
     };
 
     AccT<EPI> acc[MT][NT];
-    int const readOff = frag_offset(lane & 31, lane >> 5);
+    // byte offset, inside a 32-row block's 2 KB, of this lane's 16 bytes of fragment ks
+    int readOff[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+    {
+        if constexpr (IL)
+        {
+            readOff[ks] = ks * 1024 + frag_offset(lane & 31, lane >> 5);
+        }
+        else
+        {
+            int const fr = lane & 31, rr = fr & 15;
+            readOff[ks] = (fr >> 4) * 1024 + rr * 64 + (((ks * 2 + (lane >> 5)) ^ (rr >> 2)) << 4);
+        }
+    }
     auto multiply = [&](int slot) {
-        uint8_t const* base = lds + slot * STAGE + readOff;
+        uint8_t const* base = lds + slot * STAGE;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
         {
@@ -734,12 +765,12 @@ __device__ __forceinline__ void linear_tile_run_dma(
 #pragma unroll
             for (int i = 0; i < MT; ++i)
             {
-                fa[i] = *reinterpret_cast<i32x4 const*>(base + ((wm * MT + i) * 2 + ks) * 1024);
+                fa[i] = *reinterpret_cast<i32x4 const*>(base + (wm * MT + i) * 2048 + readOff[ks]);
             }
 #pragma unroll
             for (int j = 0; j < NT; ++j)
             {
-                fb[j] = *reinterpret_cast<i32x4 const*>(base + (AF + (wn * NT + j) * 2 + ks) * 1024);
+                fb[j] = *reinterpret_cast<i32x4 const*>(base + AF * 1024 + (wn * NT + j) * 2048 + readOff[ks]);
             }
 #pragma unroll
             for (int i = 0; i < MT; ++i)
@@ -939,7 +970,7 @@ __global__ __launch_bounds__(512) void int8_linear_persistent_kernel(LinearArgs 
 }
 
 // The persistent tile plan with direct-to-LDS loads for the 256 x 256 tiles.
-template <bool IL_OUT, int EPI>
+template <bool IL, bool IL_OUT, int EPI>
 __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[4 * 2 * (kBig / 32) * 2 * 1024];
@@ -955,7 +986,7 @@ __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p
             n0 = (int) (pan * pw + rem % pw) * kBig;
             t0 = (int) (rem / pw) * kBig;
         };
-        linear_tile_run_dma<IL_OUT, EPI>(p, count, origin, lds, sScale);
+        linear_tile_run_dma<IL, IL_OUT, EPI>(p, count, origin, lds, sScale);
     }
     else
     {
@@ -965,7 +996,7 @@ __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p
             n0 = (int) (tile % nbm) * kSmall;
             t0 = p.tokMain * kBig + (int) (tile / nbm) * kSmall;
         };
-        linear_tile_run<2, 4, 2, 1, true, true, IL_OUT, EPI>(p, 1, origin, lds, sScale);
+        linear_tile_run<2, 4, 2, 1, IL, IL, IL_OUT, EPI>(p, 1, origin, lds, sScale);
     }
 }
 
@@ -1030,11 +1061,12 @@ int launch_shape(hipStream_t stream, LinearArgs a)
             char const* e = getenv("TRTAMD_LINEAR_DIRECT");
             return e ? atoi(e) : 1;
         }();
-        if constexpr (IL_W && IL_IN && (EPI == kAFFINE || EPI == kGELU))
+        if constexpr (IL_W == IL_IN && (EPI == kAFFINE || EPI == kGELU || EPI == kF16_AFFINE || EPI == kF16_GELU))
         {
             if (direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
             {
-                hipLaunchKernelGGL((int8_linear_dma_kernel<IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0, stream, a);
+                hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0, stream,
+                    a);
                 return check_launch("int8_linear_dma_kernel");
             }
         }

@@ -189,7 +189,7 @@ def run_fp16(a, w, alpha, beta, gelu):
 
 
 @pytest.mark.parametrize("T,K,N", [(1, 32, 32), (77, 96, 64), (300, 768, 768), (519, 1024, 3072), (9000, 128, 1024),
-                                   (16500, 128, 1024)])
+                                   (16500, 128, 1024), (20000, 512, 512)])
 @pytest.mark.parametrize("gelu", [False, True])
 def test_fp16_linear(T, K, N, gelu):
     r = rng(61 + T)
