@@ -31,8 +31,6 @@ namespace trtamd
 namespace
 {
 
-constexpr float kRoundMagic = 12582912.f; // 1.5 * 2^23: adding it rounds to nearest even
-constexpr int kRoundMagicBits = 0x4B400000;
 constexpr int kBigTile = 256; // channels and tokens of the large workgroup tile
 
 enum Epilogue
@@ -94,25 +92,6 @@ __device__ inline float gelu_erf(float y)
     p = fmaf(p, a, -1.150788426e+00f);
     p = fmaf(p, a, -1.000037551e+00f);
     return fmaf(-a, __builtin_amdgcn_exp2f(p), fmaxf(y, 0.f));
-}
-
-// v = x + 1.5*2^23 already formed: clamp the bit pattern so that the low byte is sat8(rne(x)).
-__device__ inline uint32_t clamp_sat8_bits(float v)
-{
-    int const b = bits_as<int>(v);
-    return (uint32_t) min(max(b, kRoundMagicBits - 128), kRoundMagicBits + 127);
-}
-
-__device__ inline uint32_t round_sat8_bits(float v)
-{
-    return clamp_sat8_bits(v + kRoundMagic);
-}
-
-__device__ inline uint32_t low_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3)
-{
-    uint32_t const lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
-    uint32_t const hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
-    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
 // One operand fragment of v_mfma_i32_32x32x32_i8 is 32 rows x 32 k-bytes; lane l feeds row l%32,
@@ -196,26 +175,27 @@ __device__ __forceinline__ void store_block(
     }
     else
     {
+        // Results are formed as unsigned bytes, x + 128: v_cvt_pk_u8_f32 rounds to nearest even, saturates to
+        // [0, 255] and places the byte in one instruction; one XOR per dword returns to two's complement.
         int d[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g)
         {
-            uint32_t b[4];
+            uint32_t w = 0;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
             {
-                float y = fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
                 if constexpr (EPI == kGELU)
                 {
-                    // one rounding of gelu * scale + 1.5*2^23: the sum's low bits are the integer
-                    b[e] = clamp_sat8_bits(fmaf(gelu_erf(y), p.qOut, kRoundMagic));
+                    float const y = fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(gelu_erf(y), p.qOut, 128.f), e, w);
                 }
                 else
                 {
-                    b[e] = round_sat8_bits(y);
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf((float) acc[4 * g + e], al[g][e], be[g][e] + 128.f), e, w);
                 }
             }
-            d[g] = (int) low_bytes(b[0], b[1], b[2], b[3]);
+            d[g] = (int) (w ^ 0x80808080u);
         }
         // lanes l < 32 hold channels [0-3][8-11][16-19][24-27], lanes l+32 the gaps
         auto const s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);

@@ -266,8 +266,11 @@ int skip_layer_norm(hipStream_t stream, int32_t ld, int64_t n, T const* in, T co
 // epsilon 2^-10, out = sat8(rne(y * qScale)).  The statistics are exact: integer dot products of
 // the bytes (v_dot4_i32_i8) summed over the wave, the bias terms as binary32 dot products, all
 // combined in binary64.  gamma*qScale and beta*qScale of the lane's 16 channels stay in registers
-// for all rows; bytes are converted through the unsigned path (x + 128) with the offset folded into
-// the additive constant, and rounded by the 1.5*2^23 constant.
+// for all rows.  A signed byte becomes binary32 in one instruction (v_cvt_f32_i32 with a sign-extending
+// byte select); a result becomes a byte in one more: v_cvt_pk_u8_f32 rounds to nearest even, saturates to
+// [0, 255] and places the byte, so 128 is folded into beta and one XOR per dword returns to two's
+// complement.  Loads and stores are ordinary ones: in a network the tensors were just written by the layer
+// before and are read by the layer after, and the last-level cache keeps them in between.
 // ------------------------------------------------------------------------------------------
 template <int R, bool HAS_BIAS>
 __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_t const rows,
@@ -291,8 +294,8 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
         // rows past the end re-read the last row (and store nothing); idle lanes contribute zeros
         int64_t const row = min(row0 + r, rows - 1);
         int64_t const off = row * ld + ch;
-        xi[r] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(in + off));
-        xs[r] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(skip + off));
+        xi[r] = *reinterpret_cast<u32x4 const*>(in + off);
+        xs[r] = *reinterpret_cast<u32x4 const*>(skip + off);
         if (!lane_ok)
         {
             xi[r] = u32x4{0, 0, 0, 0};
@@ -315,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
         for (int k = 0; k < 8; ++k)
         {
             gq[h * 8 + k] = (float) g.e[k] * qScale;
-            bq[h * 8 + k] = (float) b.e[k] * qScale;
+            bq[h * 8 + k] = (float) b.e[k] * qScale + 128.f; // results are formed as unsigned bytes
             if (HAS_BIAS)
             {
                 float const v = lane_ok ? (float) c.e[k] : 0.f;
@@ -332,7 +335,6 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
     }
     double const dIn = (double) dqIn, dSk = (double) dqSkip;
     double const rld = 1.0 / (double) ld;
-    constexpr float kMagic = 12582912.f;
 #pragma unroll
     for (int r = 0; r < R; ++r)
     {
@@ -375,32 +377,26 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
         float const rsigma = rsqrtf(fmaxf(var, 0.f) + 0.0009765625f);
         float const a1 = dqIn * rsigma;
         float const a2 = dqSkip * rsigma;
-        float const c1 = (float) ((-128.0 * (dIn + dSk) - mean) * (double) rsigma);
+        float const c1 = (float) (-mean * (double) rsigma);
         u32x4 o;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
         {
-            uint32_t const ua = xi[r][q] ^ 0x80808080u;
-            uint32_t const us = xs[r][q] ^ 0x80808080u;
-            uint32_t yb[4];
+            uint32_t yw = 0;
 #pragma unroll
             for (int k = 0; k < 4; ++k)
             {
-                float const fa = (float) ((ua >> (8 * k)) & 0xffu);
-                float const fs = (float) ((us >> (8 * k)) & 0xffu);
+                float const fa = i8_to_f32(xi[r][q], k);
+                float const fs = i8_to_f32(xs[r][q], k);
                 float const c = HAS_BIAS ? fmaf(bs[q * 4 + k], rsigma, c1) : c1;
                 float const nrm = fmaf(fa, a1, fmaf(fs, a2, c));
-                float y = fmaf(gq[q * 4 + k], nrm, bq[q * 4 + k]);
-                y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
-                yb[k] = __float_as_uint(y + kMagic);
+                yw = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(gq[q * 4 + k], nrm, bq[q * 4 + k]), k, yw);
             }
-            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
-            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-            o[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            o[q] = yw ^ 0x80808080u;
         }
         if (lane_ok && row0 + r < rows)
         {
-            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + (row0 + r) * ld + ch));
+            *reinterpret_cast<u32x4*>(out + (row0 + r) * ld + ch) = o;
         }
     }
 }
@@ -451,14 +447,14 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
 #pragma unroll
     for (int i = 0; i < NI; ++i)
     {
-        xi[i] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(in + base + i * kStep * groupStride));
-        xs[i] = __builtin_nontemporal_load(reinterpret_cast<u32x4 const*>(skip + base + i * kStep * groupStride));
+        xi[i] = *reinterpret_cast<u32x4 const*>(in + base + i * kStep * groupStride);
+        xs[i] = *reinterpret_cast<u32x4 const*>(skip + base + i * kStep * groupStride);
     }
     // gamma/beta are staged after the tensor loads were issued, so their latency overlaps
     for (int i = threadIdx.x; i < LD; i += THREADS)
     {
         sGamma[i] = (float) gamma[i] * qScale;
-        sBeta[i] = (float) beta[i] * qScale;
+        sBeta[i] = (float) beta[i] * qScale + 128.f; // results are formed as unsigned bytes
     }
     int sIn = 0, sSk = 0, sII = 0, sIS = 0, sSS = 0;
 #pragma unroll
@@ -525,14 +521,17 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
     double const ex2 = (dIn * dIn * sII + 2.0 * dIn * dSk * sIS + dSk * dSk * sSS) * (1.0 / LD);
     float const var = (float) (ex2 - mean * mean);
     float const rsigma = rsqrtf(fmaxf(var, 0.f) + eps);
-    // bytes are read as unsigned after flipping the sign bit: u = x + 128
+    // A signed byte becomes binary32 in one instruction (v_cvt_f32_i32 with a sign-extending byte select).  Results
+    // are produced as unsigned bytes: v_cvt_pk_u8_f32 rounds to nearest even, saturates to [0, 255] and places the
+    // byte, so with 128 folded into the additive term one instruction does the rounding, the clamp to [-128, 127]
+    // and the packing, and one XOR per dword returns to two's complement.
     float const a1 = dqIn * rsigma;
     float const a2 = dqSkip * rsigma;
-    float const c1 = (float) ((-128.0 * (dIn + dSk) - mean) * (double) rsigma);
+    float const c1 = (float) (-mean * (double) rsigma);
     float const p1 = dqIn * qSkipScale;
     float const p2 = dqSkip * qSkipScale;
-    float const pc = -128.f * (dqIn + dqSkip) * qSkipScale;
-    constexpr float kMagic = 12582912.f; // 1.5 * 2^23: the sum's low mantissa byte is rne(x) in two's complement
+    float const pc = 128.f;
+    float const prelnLo = prelnMin + 128.f;
 
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -543,43 +542,34 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
 #pragma unroll
         for (int q = 0; q < 4; ++q)
         {
-            uint32_t const ua = a[q] ^ 0x80808080u;
-            uint32_t const us = s[q] ^ 0x80808080u;
             f32x4 const gq = *reinterpret_cast<f32x4 const*>(&sGamma[ch + q * 4]);
             f32x4 const bq = *reinterpret_cast<f32x4 const*>(&sBeta[ch + q * 4]);
-            uint32_t yb[4], pb[4];
+            uint32_t yw = 0, pw = 0;
 #pragma unroll
             for (int k = 0; k < 4; ++k)
             {
-                float const fa = (float) ((ua >> (8 * k)) & 0xffu);
-                float const fs = (float) ((us >> (8 * k)) & 0xffu);
+                float const fa = i8_to_f32(a[q], k);
+                float const fs = i8_to_f32(s[q], k);
                 float const nrm = fmaf(fa, a1, fmaf(fs, a2, c1));
-                float y = fmaf(gq[k], nrm, bq[k]);
-                y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
-                yb[k] = __float_as_uint(y + kMagic);
+                yw = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(gq[k], nrm, bq[k]), k, yw);
                 if (PRELN)
                 {
-                    float pv = fmaf(fa, p1, fmaf(fs, p2, pc));
-                    pv = __builtin_amdgcn_fmed3f(pv, prelnMin, 127.f);
-                    pb[k] = __float_as_uint(pv + kMagic);
+                    float const pv = fmaf(fa, p1, fmaf(fs, p2, pc));
+                    pw = __builtin_amdgcn_cvt_pk_u8_f32(fmaxf(pv, prelnLo), k, pw);
                 }
             }
-            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
-            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-            o[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            o[q] = yw ^ 0x80808080u;
             if (PRELN)
             {
-                uint32_t const plo = __builtin_amdgcn_perm(pb[1], pb[0], 0x0c0c0400u);
-                uint32_t const phi = __builtin_amdgcn_perm(pb[3], pb[2], 0x0c0c0400u);
-                po[q] = __builtin_amdgcn_perm(phi, plo, 0x05040100u);
+                po[q] = pw ^ 0x80808080u;
             }
         }
         if (valid)
         {
-            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + base + i * kStep * groupStride));
+            *reinterpret_cast<u32x4*>(out + base + i * kStep * groupStride) = o;
             if (PRELN)
             {
-                __builtin_nontemporal_store(po, reinterpret_cast<u32x4*>(preln + base + i * kStep * groupStride));
+                *reinterpret_cast<u32x4*>(preln + base + i * kStep * groupStride) = po;
             }
         }
     }

@@ -173,8 +173,42 @@ def main():
                                                          0.01, float(wl.s_skip), 20.0)))
     report(f"SkipLN int8 linear {T}x1024", t, nbytes=T * E * 3 + 2 * E * 2)
 
-    # ---- the linear layers and reformats of the BERT-large INT8 encoder, B=128, 33289 tokens -------------
+    # ---- SkipLayerNorm with nothing in the last-level cache: operands rotate through more than 256 MB -----
     Tq = 33289
+    n_sets = 12  # 12 x 3 x 34 MB = 1.2 GB
+    sets = [tuple(torch.randint(-127, 128, (32, Tq, 32), dtype=torch.int8, device="cuda") for _ in range(3))
+            for _ in range(n_sets)]
+    gh1, bh1 = dev(r.uniform(0.5, 1.5, 1024).astype(np.float16)), dev((0.1 * r.standard_normal(1024)).astype(np.float16))
+    turn = [0]
+
+    def skipln_rotating():
+        xi, si, oi = sets[turn[0] % n_sets]
+        turn[0] += 1
+        api.check(api.skipln_interleaved_large_hface(stream, 1024, Tq, xi.data_ptr(), si.data_ptr(), bh1.data_ptr(),
+                                                     gh1.data_ptr(), oi.data_ptr(), 0.02, 0.02, 30.0))
+
+    t = timeit(skipln_rotating)
+    report(f"SkipLN int8 kCHW32 {Tq}x1024, rotating 1.2 GB", t, nbytes=Tq * 1024 * 3 + 2 * 1024 * 2)
+    xi, si, oi = sets[0]
+    t = timeit(lambda: api.check(api.skipln_interleaved_large_hface(
+        stream, 1024, Tq, xi.data_ptr(), si.data_ptr(), bh1.data_ptr(), gh1.data_ptr(), oi.data_ptr(), 0.02, 0.02, 30.0)))
+    report(f"SkipLN int8 kCHW32 {Tq}x1024, same buffers", t, nbytes=Tq * 1024 * 3 + 2 * 1024 * 2)
+    del sets, xi, si, oi
+    n_sets = 6  # 6 x 3 x 100 MB
+    sets = [tuple(torch.randn((n_big, ld), dtype=torch.float16, device="cuda") for _ in range(3)) for _ in range(n_sets)]
+    turn[0] = 0
+
+    def skipln16_rotating():
+        xi, si, oi = sets[turn[0] % n_sets]
+        turn[0] += 1
+        api.check(api.skip_layer_norm_fp16(stream, ld, n_big * ld, xi.data_ptr(), si.data_ptr(), bh.data_ptr(),
+                                           gh.data_ptr(), oi.data_ptr(), biash.data_ptr()))
+
+    t = timeit(skipln16_rotating)
+    report(f"SkipLN fp16 {n_big}x768, rotating 1.8 GB", t, nbytes=n_big * ld * 3 * 2 + 3 * ld * 2)
+    del sets
+
+    # ---- the linear layers and reformats of the BERT-large INT8 encoder, B=128, 33289 tokens -------------
 
     def qnormal(shape):
         v = torch.randn(shape, device="cuda")
