@@ -217,6 +217,29 @@ __device__ inline float i8_to_f32(uint32_t w, int k)
     return (float) (int8_t) (w >> (8 * k));
 }
 
+// Global stores that write through the XCD's L2 (`sc1`, agent scope): the data leaves the L2 while the kernel runs
+// instead of in the write-back at its end, and still allocates in the last-level cache, where the kernel of the next
+// layer finds it (a non-temporal store does not).  Inline assembly, since no builtin sets this bit on a vector
+// store; the s_nop covers the wait states the hardware asks for between a store of more than 8 bytes and an
+// overwrite of its data registers, which the compiler cannot insert for an instruction it does not see.
+template <typename V>
+__device__ inline void store_through_l2(void* p, V const& v)
+{
+    static_assert(sizeof(V) == 16 || sizeof(V) == 8 || sizeof(V) == 4, "one dword, two or four");
+    if constexpr (sizeof(V) == 16)
+    {
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+    }
+    else if constexpr (sizeof(V) == 8)
+    {
+        asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    }
+    else
+    {
+        asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    }
+}
+
 // XCD-aware block remap: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so work
 // items that share data (the query tiles of one head) are renumbered to land on one XCD's L2.
 __device__ inline uint32_t xcd_remap(uint32_t bid, uint32_t nblocks)

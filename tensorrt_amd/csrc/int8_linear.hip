@@ -108,7 +108,22 @@ __device__ inline int frag_offset(int row, int half)
 // of four consecutive channels.  For the INT8 outputs the two lanes that share a token trade two packed dwords
 // (v_permlane32_swap), after which lane l holds the 16 consecutive channels 16*(l/32)..+15 and stores them with
 // one 16-byte write.
-template <bool IL_OUT, int EPI, bool FULL = false>
+// THROUGH: the store writes through the L2 (inline assembly, which the compiler's own vmcnt bookkeeping does not see:
+// only for the kernel that places its waits itself).
+template <bool THROUGH, typename V>
+__device__ __forceinline__ void store_out(void* p, V const& v)
+{
+    if constexpr (THROUGH)
+    {
+        store_through_l2(p, v);
+    }
+    else
+    {
+        *static_cast<V*>(p) = v;
+    }
+}
+
+template <bool IL_OUT, int EPI, bool FULL = false, bool THROUGH = false>
 __device__ __forceinline__ void store_block(
     LinearArgs const& p, AccT<EPI> const& acc, int const c0, int const tb, float const* sAlpha, float const* sBeta)
 {
@@ -134,7 +149,7 @@ __device__ __forceinline__ void store_block(
             for (int g = 0; g < 4; ++g)
             {
                 i32x4 const v = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
-                *reinterpret_cast<i32x4*>(static_cast<int32_t*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi) = v;
+                store_out<THROUGH>(static_cast<int32_t*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi, v);
             }
         }
     }
@@ -152,7 +167,7 @@ __device__ __forceinline__ void store_block(
                     float const y = fmaf(acc[4 * g + e], al[g][e], be[g][e]);
                     h[e] = (f16) (EPI == kF16_GELU ? gelu_erf(y) : y);
                 }
-                *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi) = h;
+                store_out<THROUGH>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi, h);
             }
         }
     }
@@ -169,7 +184,7 @@ __device__ __forceinline__ void store_block(
                 {
                     h[e] = (f16) fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
                 }
-                *reinterpret_cast<f16x4*>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi) = h;
+                store_out<THROUGH>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi, h);
             }
         }
     }
@@ -205,7 +220,7 @@ __device__ __forceinline__ void store_block(
         {
             int const c = c0 + 16 * hi;
             size_t const o = IL_OUT ? ((size_t) (c >> 5) * p.T + t) * 32 + (c & 31) : (size_t) t * p.N + c;
-            *reinterpret_cast<i32x4*>(static_cast<int8_t*>(p.out) + o) = packed;
+            store_out<THROUGH>(static_cast<int8_t*>(p.out) + o, packed);
         }
     }
 }
@@ -862,7 +877,7 @@ __device__ __forceinline__ void linear_tile_run_dma(
             for (int jj = 0; jj < NT; ++jj)
             {
                 int const cl = (wm * MT + i) * 32;
-                store_block<IL_OUT, EPI, true>(p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, scales(j & 1, 0) + cl,
+                store_block<IL_OUT, EPI, true, true>(p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, scales(j & 1, 0) + cl,
                     scales(j & 1, 1) + cl);
             }
         }

@@ -269,8 +269,9 @@ int skip_layer_norm(hipStream_t stream, int32_t ld, int64_t n, T const* in, T co
 // for all rows.  A signed byte becomes binary32 in one instruction (v_cvt_f32_i32 with a sign-extending
 // byte select); a result becomes a byte in one more: v_cvt_pk_u8_f32 rounds to nearest even, saturates to
 // [0, 255] and places the byte, so 128 is folded into beta and one XOR per dword returns to two's
-// complement.  Loads and stores are ordinary ones: in a network the tensors were just written by the layer
-// before and are read by the layer after, and the last-level cache keeps them in between.
+// complement.  Loads are ordinary ones and stores write through the L2 (not non-temporal): in a network the
+// tensors were just written by the layer before and are read by the layer after, and the last-level cache
+// keeps them in between.
 // ------------------------------------------------------------------------------------------
 template <int R, bool HAS_BIAS>
 __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_t const rows,
@@ -396,7 +397,7 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
         }
         if (lane_ok && row0 + r < rows)
         {
-            *reinterpret_cast<u32x4*>(out + (row0 + r) * ld + ch) = o;
+            store_through_l2(out + (row0 + r) * ld + ch, o);
         }
     }
 }
@@ -566,10 +567,10 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
         }
         if (valid)
         {
-            *reinterpret_cast<u32x4*>(out + base + i * kStep * groupStride) = o;
+            store_through_l2(out + base + i * kStep * groupStride, o);
             if (PRELN)
             {
-                *reinterpret_cast<u32x4*>(preln + base + i * kStep * groupStride) = po;
+                store_through_l2(preln + base + i * kStep * groupStride, po);
             }
         }
     }
