@@ -594,9 +594,7 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
                 {
                     off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
                 }
-                // agent scope: the store writes through the XCD's L2 as the kernel runs (the next layer reads it from the
-                // last-level cache) instead of in the write-back at the kernel's end
-                __hip_atomic_store(reinterpret_cast<uint32_t*>(dst + off), packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *reinterpret_cast<uint32_t*>(dst + off) = packed;
             }
         }
     }
@@ -942,9 +940,7 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
                 {
                     off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
                 }
-                // agent scope: the store writes through the XCD's L2 as the kernel runs (the next layer reads it from the
-                // last-level cache) instead of in the write-back at the kernel's end
-                __hip_atomic_store(reinterpret_cast<uint32_t*>(dst + off), packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *reinterpret_cast<uint32_t*>(dst + off) = packed;
             }
         }
     }

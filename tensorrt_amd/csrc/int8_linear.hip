@@ -109,7 +109,8 @@ __device__ inline int frag_offset(int row, int half)
 // (v_permlane32_swap), after which lane l holds the 16 consecutive channels 16*(l/32)..+15 and stores them with
 // one 16-byte write.
 // THROUGH: the store writes through the L2 (inline assembly, which the compiler's own vmcnt bookkeeping does not see:
-// only for the kernel that places its waits itself).
+// only for the kernel that places its waits itself, and only where a wavefront's store covers whole cache lines, the
+// 32-interleaved INT8 output: 32 tokens x 32 bytes; narrower pieces are better merged in the L2 first).
 template <bool THROUGH, typename V>
 __device__ __forceinline__ void store_out(void* p, V const& v)
 {
@@ -877,7 +878,7 @@ __device__ __forceinline__ void linear_tile_run_dma(
             for (int jj = 0; jj < NT; ++jj)
             {
                 int const cl = (wm * MT + i) * 32;
-                store_block<IL_OUT, EPI, true, true>(p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, scales(j & 1, 0) + cl,
+                store_block<IL_OUT, EPI, true, IL_OUT && (EPI == kAFFINE || EPI == kGELU)>(p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, scales(j & 1, 0) + cl,
                     scales(j & 1, 1) + cl);
             }
         }
