@@ -38,7 +38,7 @@ PEAK_HBM = 8.0e12        # B/s
 MHA_TRAFFIC_BYTES = 75_200_000
 LN_TRAFFIC_BYTES = 59_700_000
 # the same for the encoder workload's defaults (B=128, lengths uniform[128,384], seed 1: 33289 tokens)
-ENC_FFN1_TRAFFIC_BYTES = 325_000_000
+ENC_FFN1_TRAFFIC_BYTES = 240_000_000
 ENC_MHA_TRAFFIC_BYTES = 137_700_000
 ENC_LN_TRAFFIC_BYTES = 108_800_000
 
