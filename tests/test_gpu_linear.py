@@ -1,8 +1,9 @@
 """INT8 linear layer on the GPU against the CPU oracle, through the C-ABI.
 
-Bar: INT32 accumulators bit-exact; requantised INT8 within 1 LSB (the affine epilogue is the same
-single fmaf on both sides and is expected to agree exactly; the GELU epilogue evaluates erf by a
-rational approximation on the GPU and in binary64 in the oracle); FP16 output within the
+Bar: INT32 accumulators bit-exact; requantised INT8 within 1 LSB (the affine epilogue is a single
+fmaf on both sides, the GPU's with 128 folded into the addend because it forms the byte unsigned, so
+the two agree except for results within a rounding error of a tie; the GELU epilogue evaluates erf
+through a polynomial on the GPU and in binary64 in the oracle); FP16 output within the
 floating-point tolerance.
 """
 import ctypes as C
@@ -90,6 +91,27 @@ def test_affine_int8(T, K, N, a_il, out_il):
     ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE, out_interleaved=out_il)
     assert (np.abs(ref.astype(int)) == 127).any() or (ref == -128).any(), "inputs should exercise saturation"
     assert_int8_close(got, ref, what="affine", max_frac_off=1e-3)
+
+
+@pytest.mark.parametrize("il", [False, True])
+@pytest.mark.parametrize("T,K,N", [(255, 64, 32), (512, 256, 256)])
+def test_requantisation_ties_and_saturation_are_exact(T, K, N, il):
+    """Accumulators -127..127 times scales that are multiples of 1/2: every product is exact in binary32,
+    half of them lie on a tie (round to even) and the large scales run into both ends of the INT8 range, so
+    the expected bytes follow from integer arithmetic alone."""
+    a = np.zeros((T, K), np.int8)
+    a[:, 0] = (np.arange(T) % 255 - 127).astype(np.int8)
+    w = np.zeros((N, K), np.int8)
+    w[:, 0] = 1
+    alpha = (0.5 * (1 + np.arange(N) % 7)).astype(np.float32)     # 0.5 .. 3.5
+    beta = (0.5 * (np.arange(N) % 5) - 1.0).astype(np.float32)    # -1 .. 1 in halves
+    got = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=il, out_il=il, w_il=il)
+    y = a[:, :1].astype(np.float64) * alpha[None, :].astype(np.float64) + beta[None, :].astype(np.float64)
+    want = np.clip(np.rint(y), -128, 127).astype(np.int8)          # numpy's rint rounds ties to even
+    assert (np.abs(y - np.floor(y)) == 0.5).any() and (want == 127).any() and (want == -128).any()
+    if il:
+        want = interleave(want)
+    assert np.array_equal(got, want)
 
 
 @pytest.mark.parametrize("T,K,N", [(17, 64, 32), (519, 1024, 1024), (700, 1024, 4096)])
