@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBlock) void embln_kernel(int const ld, int const B
             cnt += ok ? (float) VPT : 0.f;
             if (MODE == kMTRON && ok)
             {
-                *reinterpret_cast<u32x4*>(skipOut + tokenIdx * ld + (int64_t) (lane + kWaveSize * j) * VPT) = pre.u;
+                store_through_l2(skipOut + tokenIdx * ld + (int64_t) (lane + kWaveSize * j) * VPT, pre.u);
             }
         }
         Welford st;
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kBlock) void embln_kernel(int const ld, int const B
                 {
                     y.e[k] = (T) (gk[j][k] * (v[j][k] - mu) * rsigma + bk[j][k]);
                 }
-                *reinterpret_cast<u32x4*>(output + tokenIdx * ld + (int64_t) vi * VPT) = y.u;
+                store_through_l2(output + tokenIdx * ld + (int64_t) vi * VPT, y.u);
             }
         }
     }

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(kBlock) void skipln_rows_kernel(int const ld, int64
                 {
                     y.e[k] = (T) ((float) g[j].e[k] * (v[j][k] - mu) * rsigma + (float) b[j].e[k]);
                 }
-                *reinterpret_cast<u32x4*>(out + (row0 + r) * ld + (int64_t) vi * VPT) = y.u;
+                store_through_l2(out + (row0 + r) * ld + (int64_t) vi * VPT, y.u);
             }
         }
     }
