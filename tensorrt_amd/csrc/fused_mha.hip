@@ -913,35 +913,52 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
 
         // ---- out8 = sat8(rne(acc2 * scale_bmm2)): binary32 product (rounded on its own, not fused
         //      into the add), rounded to an integer through the magic constant, clamped on the bit
-        //      patterns (monotone for the positive results; anything negative is below the range)
+        //      patterns (monotone for the positive results; anything negative is below the range).
+        //      Lane (g, query) then holds bytes 4g..4g+3 of each 16-byte quarter dt of the query's row; a 4 x 4
+        //      transpose over the four rows of 16 lanes (v_permlane32_swap, v_permlane16_swap) leaves it with the
+        //      whole quarter dt = g, which goes out as one 16-byte store.
+        uint32_t pk[4];
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+        {
+            uint32_t yb[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                int const bits = __float_as_int(mul_rounded((float) oacc[dt][j], a.scaleBmm2) + kMagic);
+                yb[j] = (uint32_t) min(max(bits, kMagicBits - 128), kMagicBits + 127);
+            }
+            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+            pk[dt] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+        {
+            // rows 0,1 keep quarter 0 / 1 of their own and get the same quarter of rows 2,3; rows 2,3 the other way
+            auto const s02 = __builtin_amdgcn_permlane32_swap(pk[0], pk[2], false, false);
+            auto const s13 = __builtin_amdgcn_permlane32_swap(pk[1], pk[3], false, false);
+            // even rows keep the first of a pair and get it from the odd row below; odd rows the second
+            auto const t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+            auto const t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+            pk[0] = t01[0];
+            pk[1] = t01[1];
+            pk[2] = t23[0];
+            pk[3] = t23[1];
+        }
         if (qValid)
         {
             uint8_t* dst = static_cast<uint8_t*>(a.out);
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            int const d0 = g * 16;
+            int64_t off;
+            if (INTERLEAVED)
             {
-                uint32_t yb[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    int const bits = __float_as_int(mul_rounded((float) oacc[dt][j], a.scaleBmm2) + kMagic);
-                    yb[j] = (uint32_t) min(max(bits, kMagicBits - 128), kMagicBits + 127);
-                }
-                uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
-                uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-                uint32_t const packed = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                int const d0 = dt * 16 + g * 4;
-                int64_t off;
-                if (INTERLEAVED)
-                {
-                    off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
-                }
-                else
-                {
-                    off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
-                }
-                *reinterpret_cast<uint32_t*>(dst + off) = packed;
+                off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
             }
+            else
+            {
+                off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
+            }
+            u32x4 const quarter = {pk[0], pk[1], pk[2], pk[3]};
+            *reinterpret_cast<u32x4*>(dst + off) = quarter;
         }
     }
 }
