@@ -1445,10 +1445,12 @@ __device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq,
             }
         }
 
-        if (qValid)
+        // Lane (g, query) holds 8 bytes of each 32-byte quarter dt of the query's 128-byte row; a 4 x 4 transpose over
+        // the four rows of 16 lanes (v_permlane32_swap, v_permlane16_swap, once for each dword) leaves it with the
+        // whole quarter dt = g, which goes out as two 16-byte stores.
         {
             float const rinv = 1.f / sacc[0];
-            uint8_t* dst = static_cast<uint8_t*>(a.out);
+            uint32_t lo[4], hi[4];
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
             {
@@ -1458,10 +1460,31 @@ __device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq,
                 {
                     y[j] = (f16) (oacc[dt][j] * rinv);
                 }
-                int const d0 = dt * 16 + g * 4;
+                u32x2 const w = __builtin_bit_cast(u32x2, y);
+                lo[dt] = w[0];
+                hi[dt] = w[1];
+            }
+            auto const rows_transpose = [](uint32_t(&x)[4]) {
+                auto const s02 = __builtin_amdgcn_permlane32_swap(x[0], x[2], false, false);
+                auto const s13 = __builtin_amdgcn_permlane32_swap(x[1], x[3], false, false);
+                auto const t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+                auto const t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+                x[0] = t01[0];
+                x[1] = t01[1];
+                x[2] = t23[0];
+                x[3] = t23[1];
+            };
+            rows_transpose(lo);
+            rows_transpose(hi);
+            if (qValid)
+            {
+                uint8_t* dst = static_cast<uint8_t*>(a.out);
                 int64_t const off
-                    = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + d0) * 2;
-                *reinterpret_cast<u32x2*>(dst + off) = __builtin_bit_cast(u32x2, y);
+                    = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + g * 16) * 2;
+                u32x4 const first = {lo[0], hi[0], lo[1], hi[1]};
+                u32x4 const second = {lo[2], hi[2], lo[3], hi[3]};
+                *reinterpret_cast<u32x4*>(dst + off) = first;
+                *reinterpret_cast<u32x4*>(dst + off + 16) = second;
             }
         }
     }
