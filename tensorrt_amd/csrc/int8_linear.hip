@@ -154,39 +154,34 @@ __device__ __forceinline__ void store_block(
             }
         }
     }
-    else if constexpr (EPI >= kF16_AFFINE)
+    else if constexpr (EPI >= kF16_AFFINE || EPI == kHALF)
     {
-        if (live)
+        u32x2 w[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
         {
+            f16x4 h;
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
+            for (int e = 0; e < 4; ++e)
             {
-                f16x4 h;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                {
-                    float const y = fmaf(acc[4 * g + e], al[g][e], be[g][e]);
-                    h[e] = (f16) (EPI == kF16_GELU ? gelu_erf(y) : y);
-                }
-                store_out<THROUGH>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi, h);
+                float const y = fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
+                h[e] = (f16) (EPI == kF16_GELU ? gelu_erf(y) : y);
             }
+            w[g] = __builtin_bit_cast(u32x2, h);
         }
-    }
-    else if constexpr (EPI == kHALF)
-    {
+        // lanes l < 32 hold channels 8g..8g+3 of each group g, lanes l+32 the other four: after the swaps lane l has
+        // groups 0 and 1 whole, lane l+32 groups 2 and 3: 16 consecutive channels, two 16-byte stores
+        auto const a0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[2][0], false, false);
+        auto const a1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[2][1], false, false);
+        auto const b0 = __builtin_amdgcn_permlane32_swap(w[1][0], w[3][0], false, false);
+        auto const b1 = __builtin_amdgcn_permlane32_swap(w[1][1], w[3][1], false, false);
+        u32x4 const first = {a0[0], a1[0], a0[1], a1[1]};
+        u32x4 const second = {b0[0], b1[0], b0[1], b1[1]};
         if (live)
         {
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-            {
-                f16x4 h;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                {
-                    h[e] = (f16) fmaf((float) acc[4 * g + e], al[g][e], be[g][e]);
-                }
-                store_out<THROUGH>(static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 8 * g + 4 * hi, h);
-            }
+            f16* dst = static_cast<f16*>(p.out) + (size_t) t * p.N + c0 + 16 * hi;
+            store_out<THROUGH>(dst, first);
+            store_out<THROUGH>(dst + 8, second);
         }
     }
     else
@@ -675,8 +670,8 @@ __device__ __forceinline__ void linear_tile_run_dma(
     constexpr int LB = BF / NWAVES;
     constexpr int STAGE = (AF + BF) * 1024;
     constexpr int kLoads = LA + LB;           // direct loads per wavefront and stage
-    // global stores per wavefront in a tile's epilogue: one 16-byte store per accumulator block (INT8), four of 8 bytes (FP16)
-    constexpr int kStores = MT * NT * (EPI >= kF16_AFFINE ? 4 : 1);
+    // global stores per wavefront in a tile's epilogue: one 16-byte store per accumulator block (INT8), two (FP16)
+    constexpr int kStores = MT * NT * (EPI >= kF16_AFFINE ? 2 : 1);
     static_assert(EPI == kAFFINE || EPI == kGELU || EPI == kF16_AFFINE || EPI == kF16_GELU, "store count per block");
 
     int const lane = threadIdx.x & 63;
