@@ -54,6 +54,23 @@ __device__ inline float mul_rounded(float a, float b)
     return a * b;
 }
 
+// x[dt] of the lane in 16-lane row g  ->  x[g'] = what row g' held in its x[g]: a 4 x 4 transpose over the four rows of
+// a wavefront.  All 64 lanes must be active.  The attention kernels end with lane (g, query) holding a piece of each
+// quarter dt of the query's output row; transposed, it holds the whole quarter dt = g and stores it in one piece.
+__device__ inline void rows_transpose(uint32_t (&x)[4])
+{
+    // rows 0,1 keep x[0] / x[1] of their own and get the same from rows 2,3; rows 2,3 the other way round
+    auto const s02 = __builtin_amdgcn_permlane32_swap(x[0], x[2], false, false);
+    auto const s13 = __builtin_amdgcn_permlane32_swap(x[1], x[3], false, false);
+    // even rows keep the first of a pair and get it from the odd row below them; odd rows the second
+    auto const t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+    auto const t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+    x[0] = t01[0];
+    x[1] = t01[1];
+    x[2] = t23[0];
+    x[3] = t23[1];
+}
+
 struct FmhaArgs
 {
     void const* qkv;
@@ -565,37 +582,41 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
             }
         }
 
-        // ---- out8 = sat8(rne(acc2 * scale_bmm2)); lane holds d = 16dt + 4g .. +3 of query q --
+        // ---- out8 = sat8(rne(acc2 * scale_bmm2)); lane holds d = 16dt + 4g .. +3 of query q, after the transpose
+        //      the whole quarter d = 16g .. 16g+15
+        uint32_t pk[4];
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+        {
+            uint32_t yb[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                float y = (float) oacc[dt][j] * a.scaleBmm2;
+                y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
+                yb[j] = __float_as_uint(y + kMagic);
+            }
+            uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+            uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+            pk[dt] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+        rows_transpose(pk);
         if (qValid)
         {
             uint8_t* dst = static_cast<uint8_t*>(a.out);
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+            int const d0 = g * 16;
+            int64_t off;
+            if (INTERLEAVED)
             {
-                uint32_t yb[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    float y = (float) oacc[dt][j] * a.scaleBmm2;
-                    y = __builtin_amdgcn_fmed3f(y, -128.f, 127.f);
-                    yb[j] = __float_as_uint(y + kMagic);
-                }
-                uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
-                uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-                uint32_t const packed = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                int const d0 = dt * 16 + g * 4;
-                int64_t off;
-                if (INTERLEAVED)
-                {
-                    // [N][d/32][T][32]
-                    off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
-                }
-                else
-                {
-                    off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
-                }
-                *reinterpret_cast<uint32_t*>(dst + off) = packed;
+                // [N][d/32][T][32]
+                off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
             }
+            else
+            {
+                off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
+            }
+            u32x4 const quarter = {pk[0], pk[1], pk[2], pk[3]};
+            *reinterpret_cast<u32x4*>(dst + off) = quarter;
         }
     }
 }
@@ -932,18 +953,7 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
             uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
             pk[dt] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
         }
-        {
-            // rows 0,1 keep quarter 0 / 1 of their own and get the same quarter of rows 2,3; rows 2,3 the other way
-            auto const s02 = __builtin_amdgcn_permlane32_swap(pk[0], pk[2], false, false);
-            auto const s13 = __builtin_amdgcn_permlane32_swap(pk[1], pk[3], false, false);
-            // even rows keep the first of a pair and get it from the odd row below; odd rows the second
-            auto const t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
-            auto const t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
-            pk[0] = t01[0];
-            pk[1] = t01[1];
-            pk[2] = t23[0];
-            pk[3] = t23[1];
-        }
+        rows_transpose(pk);
         if (qValid)
         {
             uint8_t* dst = static_cast<uint8_t*>(a.out);
@@ -1223,10 +1233,9 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
             }
         }
 
-        if (qValid)
         {
             float const rinv = sacc[0] > 0.f ? 1.f / sacc[0] : 0.f;
-            uint8_t* dst = static_cast<uint8_t*>(a.out);
+            uint32_t lo[4], hi[4];
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
             {
@@ -1236,10 +1245,21 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
                 {
                     y[j] = (f16) (oacc[dt][j] * rinv);
                 }
-                int const d0 = dt * 16 + g * 4;
+                u32x2 const w = __builtin_bit_cast(u32x2, y);
+                lo[dt] = w[0];
+                hi[dt] = w[1];
+            }
+            rows_transpose(lo);
+            rows_transpose(hi);
+            if (qValid)
+            {
+                uint8_t* dst = static_cast<uint8_t*>(a.out);
                 int64_t const off
-                    = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + d0) * 2;
-                *reinterpret_cast<u32x2*>(dst + off) = __builtin_bit_cast(u32x2, y);
+                    = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + ((int64_t) n * kHeadSize + g * 16) * 2;
+                u32x4 const first = {lo[0], hi[0], lo[1], hi[1]};
+                u32x4 const second = {lo[2], hi[2], lo[3], hi[3]};
+                *reinterpret_cast<u32x4*>(dst + off) = first;
+                *reinterpret_cast<u32x4*>(dst + off + 16) = second;
             }
         }
     }
@@ -1464,16 +1484,6 @@ __device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq,
                 lo[dt] = w[0];
                 hi[dt] = w[1];
             }
-            auto const rows_transpose = [](uint32_t(&x)[4]) {
-                auto const s02 = __builtin_amdgcn_permlane32_swap(x[0], x[2], false, false);
-                auto const s13 = __builtin_amdgcn_permlane32_swap(x[1], x[3], false, false);
-                auto const t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
-                auto const t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
-                x[0] = t01[0];
-                x[1] = t01[1];
-                x[2] = t23[0];
-                x[3] = t23[1];
-            };
             rows_transpose(lo);
             rows_transpose(hi);
             if (qValid)
