@@ -159,6 +159,41 @@ def test_large_problems_mix_both_tile_sizes(T, K, N):
     assert_int8_close(got_mixed, ref_mixed, what="affine, interleaved operands, linear output", max_frac_off=1e-3)
 
 
+def _random_cases(n, seed):
+    r = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        T = int(r.choice([int(r.integers(1, 300)), int(r.integers(300, 3000)), int(r.integers(8000, 12000))]))
+        K = 64 * int(r.integers(1, 17))
+        N = 32 * int(r.integers(1, 33))
+        il = bool(r.integers(0, 2))
+        out_il = bool(r.integers(0, 2))
+        epi = int(r.integers(0, 3))   # affine, gelu, fp16 output
+        cases.append((T, K, N, il, out_il, epi))
+    return cases
+
+
+@pytest.mark.parametrize("T,K,N,il,out_il,epi", _random_cases(20, 20240611))
+def test_random_shapes_layouts_and_epilogues(T, K, N, il, out_il, epi):
+    """Seeded random draws over the token count (a few rows to several rounds of tiles), K, N, operand and output
+    layouts and epilogues: whatever tile plan and kernel variant a shape selects must agree with the oracle."""
+    a, w, alpha, beta = problem(1000 + T + K + N, T, K, N)
+    if epi == 0:
+        got = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=il, w_il=il, out_il=out_il)
+        ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE, out_interleaved=out_il)
+        assert_int8_close(got, ref, what="affine", max_frac_off=1e-3)
+    elif epi == 1:
+        alpha = (alpha * 0.06).astype(np.float32)
+        beta = (beta * 0.02).astype(np.float32)
+        got = run_gpu(a, w, alpha, beta, capi.LINEAR_GELU, out_scale=31.75, a_il=il, w_il=il, out_il=out_il)
+        ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_GELU, out_scale=31.75, out_interleaved=out_il)
+        assert_int8_close(got, ref, what="gelu", max_frac_off=2e-3)
+    else:
+        got = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE_FP16, a_il=il, w_il=il)
+        ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE_FP16)
+        assert_fp_close(got, ref, what="fp16 output")
+
+
 def test_output_untouched_beyond_the_problem():
     """Rows beyond T and the bytes of neighbouring allocations are never written."""
     import torch
