@@ -183,6 +183,12 @@ typedef struct trtamd_fmha_params
  * one launch computes softmax(Q K^T * scale) V for every (sequence, head).
  * data_type: 1 = FP16, 2 = INT8 (nvinfer1::DataType values). */
 TRTAMD_API int trtamd_fused_mha_run(trtamd_stream_t stream, int32_t data_type, trtamd_fmha_params const* params);
+/* TFusedMultiHeadAttentionXMMAKernel::loadXMMAKernels
+ * (plugin/bertQKVToContextPlugin/fused_multihead_attention/fused_multihead_attention.h:63-147), which loads every
+ * kernel and raises its dynamic shared-memory limit when a runner is created: reserves the LDS of every fused
+ * kernel of this library on the current device, so that trtamd_fused_mha_run only ever launches (the first launch
+ * of a kernel otherwise does its own reservation).  Needs a GPU; idempotent. */
+TRTAMD_API int trtamd_fused_mha_prepare(void);
 /* isValid(headSize, s) of the same classes: 1 when a fused kernel covers (d, s). */
 TRTAMD_API int trtamd_fused_mha_is_valid(int32_t data_type, int32_t d, int32_t s);
 

@@ -102,6 +102,7 @@ _SIGS = {
     "trtamd_unfused_mha": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p, c_p]),
     "trtamd_fused_mha_run": (C.c_int, [c_p, i32, C.POINTER(FmhaParams)]),
     "trtamd_fused_mha_run_debug": (C.c_int, [c_p, i32, C.POINTER(FmhaParams), c_p, c_p]),
+    "trtamd_fused_mha_prepare": (C.c_int, []),
     "trtamd_fused_mha_is_valid": (C.c_int, [i32, i32, i32]),
     "trtamd_zero_padding_2d": (C.c_int, [c_p, i32, c_p, i32, i32, c_p]),
     "trtamd_int8_linear": (C.c_int, [c_p, C.POINTER(Int8LinearParams)]),
@@ -118,14 +119,16 @@ _SIGS = {
     "trtamd_dequantize_interleaved_to_fp16": (C.c_int, [c_p, i32, i32, c_p, f32, c_p]),
 }
 
-# Entry points declared in include/trtamd_bert_kernels.h (the debug hook is extra).
+# Entry points declared in include/trtamd_test_hooks.h (test-only).
+TEST_HOOK_SYMBOLS = ["trtamd_fused_mha_run_debug"]
+# Entry points declared in include/trtamd_bert_kernels.h are the rest of the table.
 # Entry points declared in include/trtamd_encoder_ops.h.
 ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear", "trtamd_fp16_linear", "trtamd_int8_linear_to_interleaved", "trtamd_int8_interleaved_to_linear",
                        "trtamd_quantize_fp16_to_interleaved", "trtamd_dequantize_interleaved_to_fp16"]
 # Entry points declared in include/trtamd_encoder_runtime.h.
 ENCODER_RUNTIME_SYMBOLS = ["trtamd_encoder_create", "trtamd_encoder_destroy", "trtamd_encoder_set_embedding",
                            "trtamd_encoder_set_layer", "trtamd_encoder_workspace_size", "trtamd_encoder_enqueue"]
-HEADER_SYMBOLS = [k for k in _SIGS if k != "trtamd_fused_mha_run_debug" and k not in ENCODER_OPS_SYMBOLS
+HEADER_SYMBOLS = [k for k in _SIGS if k not in TEST_HOOK_SYMBOLS and k not in ENCODER_OPS_SYMBOLS
                   and k not in ENCODER_RUNTIME_SYMBOLS]
 
 

@@ -23,6 +23,7 @@
 // Queries beyond the sequence length are neither computed nor written.
 #include "device_utils.hpp"
 #include "host_utils.hpp"
+#include "trtamd_test_hooks.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -1572,31 +1573,38 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_prefix_kernel(F
 // host side
 // ------------------------------------------------------------------------------------------
 
+// Raising the dynamic LDS limit is a per-function attribute, set once per process and kernel: at the first launch,
+// or ahead of it by trtamd_fused_mha_prepare.
+int ensure_lds(void const* key, char const* name, int ldsBytes)
+{
+    static std::mutex mtx;
+    static std::vector<void const*> done;
+    std::lock_guard<std::mutex> lock(mtx);
+    for (void const* p : done)
+    {
+        if (p == key)
+        {
+            return TRTAMD_STATUS_SUCCESS;
+        }
+    }
+    hipError_t const e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+    if (e != hipSuccess)
+    {
+        (void) hipGetLastError();
+        return set_error(TRTAMD_STATUS_FAILURE, "%s: cannot reserve %d bytes of LDS: %s", name, ldsBytes,
+            hipGetErrorString(e));
+    }
+    done.push_back(key);
+    return TRTAMD_STATUS_SUCCESS;
+}
+
 template <typename K>
 int launch_fmha(K kernel, char const* name, hipStream_t stream, FmhaArgs const& args, int ldsBytes, int waves)
 {
-    // Raising the dynamic LDS limit is a per-function attribute; set once per process.
-    static std::mutex mtx;
-    static std::vector<void const*> done;
+    int const st = ensure_lds(reinterpret_cast<void const*>(kernel), name, ldsBytes);
+    if (st != TRTAMD_STATUS_SUCCESS)
     {
-        std::lock_guard<std::mutex> lock(mtx);
-        void const* key = reinterpret_cast<void const*>(kernel);
-        bool found = false;
-        for (void const* p : done)
-        {
-            found = found || p == key;
-        }
-        if (!found)
-        {
-            hipError_t const e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
-            if (e != hipSuccess)
-            {
-                (void) hipGetLastError();
-                return set_error(TRTAMD_STATUS_FAILURE, "%s: cannot reserve %d bytes of LDS: %s", name, ldsBytes,
-                    hipGetErrorString(e));
-            }
-            done.push_back(key);
-        }
+        return st;
     }
     unsigned const blocks = (unsigned) args.B * args.N * args.qSplit;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWaveSize), ldsBytes, stream, args);
@@ -1704,6 +1712,23 @@ int run_f16(hipStream_t stream, FmhaArgs const& a)
     }
 #undef TRTAMD_F16
     return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "fused MHA: sequence length %d exceeds 512", a.S);
+}
+
+// Every shipped kernel's LDS reservation, so that no later launch has anything to set up.
+template <int KT>
+int prepare_kt()
+{
+    int st = ensure_lds(reinterpret_cast<void const*>(fmha_i8_prefix_kernel<KT, true, false>), "fmha_i8_prefix_interleaved",
+        Lds<1>::total(KT));
+    st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_i8_prefix_kernel<KT, false, false>), "fmha_i8_prefix",
+                      Lds<1>::total(KT));
+    st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_i8_kernel<KT, true, false>), "fmha_i8_interleaved",
+                      Lds<1>::total(KT));
+    st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_i8_kernel<KT, false, false>), "fmha_i8", Lds<1>::total(KT));
+    st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_f16_prefix_kernel<KT, false>), "fmha_f16_prefix",
+                      Lds<2>::total(KT));
+    st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_f16_kernel<KT, false>), "fmha_f16", Lds<2>::total(KT));
+    return st;
 }
 
 float bits_to_float(uint32_t u)
@@ -1902,12 +1927,23 @@ extern "C" int trtamd_fused_mha_run(trtamd_stream_t stream, int32_t data_type, t
     return fused_mha_run(as_stream(stream), data_type, params, nullptr, nullptr);
 }
 
-// Test hook: same launch, additionally dumping the first GEMM's accumulators ([b][h][s][s],
-// int32 for INT8, binary32 bit patterns for FP16) and, for INT8, the quantised probabilities.
-extern "C" TRTAMD_API int trtamd_fused_mha_run_debug(trtamd_stream_t stream, int32_t data_type,
+// Test hook (include/trtamd_test_hooks.h): same launch, additionally dumping the first GEMM's accumulators
+// ([b][h][s][s], int32 for INT8, binary32 bit patterns for FP16) and, for INT8, the quantised probabilities.
+extern "C" int trtamd_fused_mha_run_debug(trtamd_stream_t stream, int32_t data_type,
     trtamd_fmha_params const* params, int32_t* acc1, int8_t* p8)
 {
     return fused_mha_run(as_stream(stream), data_type, params, acc1, p8);
+}
+
+extern "C" int trtamd_fused_mha_prepare(void)
+{
+    int st = prepare_kt<1>();
+    st = st ? st : prepare_kt<2>();
+    st = st ? st : prepare_kt<3>();
+    st = st ? st : prepare_kt<4>();
+    st = st ? st : prepare_kt<6>();
+    st = st ? st : prepare_kt<8>();
+    return st;
 }
 
 extern "C" int trtamd_fused_mha_is_valid(int32_t data_type, int32_t d, int32_t s)

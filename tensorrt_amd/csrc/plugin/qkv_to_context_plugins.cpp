@@ -73,8 +73,12 @@ struct RunnerState
         buf.resize(v.size() * sizeof(int32_t));
         std::memcpy(buf.data(), v.data(), buf.size());
     }
-    void deserialize(void const* data)
+    // `bytes` = length of the serialised field; a negative value means "not known" (clones, whose buffer was
+    // written by serialize() a line earlier)
+    void deserialize(void const* data, int64_t bytes = -1)
     {
+        TRTAMD_VALIDATE_MSG(bytes < 0 || static_cast<size_t>(bytes) >= serializedSize(),
+            "runnerStateBuffer is shorter than the runner state it must hold");
         auto const* v = static_cast<int32_t const*>(data);
         if (unfused)
         {
@@ -109,6 +113,16 @@ bool fusedV1Valid(DataType type, int32_t headSize, int32_t S)
         return S == 128 || S == 384;
     }
     return false;
+}
+
+// What creating a fused runner does in the reference (getXMMAKernels / getXMMAKernelsV2 load every kernel and raise
+// its shared-memory limit, fused_multihead_attention.h:63-147): afterwards enqueue only launches.
+void prepareFusedKernels()
+{
+    if (deviceAvailable())
+    {
+        checkKernelStatus(trtamd_fused_mha_prepare(), "fused attention kernels");
+    }
 }
 
 void fillInt8Scales(trtamd_fmha_params& p, float scaleQkv, float scaleCtx, float rsqrtHeadSize, float dqProbs)
@@ -162,11 +176,13 @@ public:
     {
         mSM = getSmVersion();
         mUnfused.unfused = true;
+        prepareFusedKernels();
     }
 
     // runtime-phase constructor (deserialised engine)
     QkvToContextPlugin(std::string const& name, DataType type, int32_t S, int32_t B, int32_t SM, int32_t hiddenSize,
-        int32_t numHeads, float dqProbs, bool hasMask, bool hasUnfusedDispatcher, void const* runnerState)
+        int32_t numHeads, float dqProbs, bool hasMask, bool hasUnfusedDispatcher, void const* runnerState,
+        int64_t runnerStateBytes = -1)
         : QkvToContextPlugin(name, type, hiddenSize, numHeads, dqProbs, hasMask)
     {
         mS = S;
@@ -175,7 +191,7 @@ public:
         if (hasUnfusedDispatcher)
         {
             TRTAMD_VALIDATE(runnerState != nullptr);
-            mUnfused.deserialize(runnerState);
+            mUnfused.deserialize(runnerState, runnerStateBytes);
         }
     }
 
@@ -433,6 +449,7 @@ struct QkvCommonFields
     float dqProbs{-1.F};
     int32_t s{-1}, b{-1};
     void const* runnerState{nullptr};
+    int64_t runnerStateBytes{-1};
 
     void read(PluginFieldCollection const* fc, TensorRTPhase phase)
     {
@@ -471,6 +488,7 @@ struct QkvCommonFields
         if (PluginField const* f = findField(fc, "runnerStateBuffer"))
         {
             runnerState = f->data;
+            runnerStateBytes = f->length;
         }
         if (static_cast<DataType>(typeId) == DataType::kINT8 && dqProbs < 0)
         {
@@ -534,7 +552,7 @@ protected:
             TRTAMD_VALIDATE_MSG(c.runnerState == nullptr, "invalid runnerStateBuffer during runtime plugin creation");
         }
         return std::make_unique<QkvToContextPlugin>(name, type, c.s, c.b, sm, c.hiddenSize, c.numHeads, c.dqProbs,
-            c.hasMask, hasUnfused == 1, c.runnerState);
+            c.hasMask, hasUnfused == 1, c.runnerState, c.runnerStateBytes);
     }
 };
 
@@ -571,16 +589,18 @@ public:
             TRTAMD_VALIDATE(mType != DataType::kINT8);
         }
         mRunner.unfused = !varSeqlen;
+        prepareFusedKernels();
     }
 
     QkvToContextVarSeqlenPlugin(std::string const& name, int32_t S, int32_t B, DataType type, int32_t hiddenSize,
-        int32_t numHeads, float dqProbs, bool hasMask, bool varSeqlen, bool useInt8ScaleMax, void const* runnerState)
+        int32_t numHeads, float dqProbs, bool hasMask, bool varSeqlen, bool useInt8ScaleMax, void const* runnerState,
+        int64_t runnerStateBytes = -1)
         : QkvToContextVarSeqlenPlugin(name, type, hiddenSize, numHeads, dqProbs, hasMask, varSeqlen, useInt8ScaleMax)
     {
         mS = S;
         mB = B;
         TRTAMD_VALIDATE(runnerState != nullptr);
-        mRunner.deserialize(runnerState);
+        mRunner.deserialize(runnerState, runnerStateBytes);
     }
 
 protected:
@@ -919,7 +939,7 @@ protected:
         TRTAMD_VALIDATE_MSG(c.b != -1, "invalid B during runtime plugin creation");
         TRTAMD_VALIDATE_MSG(c.runnerState != nullptr, "invalid runnerStateBuffer during runtime plugin creation");
         return std::make_unique<QkvToContextVarSeqlenPlugin>(name, c.s, c.b, type, c.hiddenSize, c.numHeads, c.dqProbs,
-            c.hasMask, varSeqlen != 0, useInt8ScaleMax != 0, c.runnerState);
+            c.hasMask, varSeqlen != 0, useInt8ScaleMax != 0, c.runnerState, c.runnerStateBytes);
     }
 };
 
@@ -942,6 +962,7 @@ public:
         , mCtxScale(ctxScale)
     {
         mSM = getSmVersion();
+        prepareFusedKernels();
     }
 
 protected:

@@ -250,7 +250,11 @@ private:
 class SkipLayerNormInterleavedPlugin final : public BertPluginBase
 {
 public:
-    SkipLayerNormInterleavedPlugin(std::string const& name, bool mtron, Weights const& beta, Weights const& gamma)
+    // onDevice: put gamma and beta on the device now.  Runtime-phase objects (and their clones) do, so that neither
+    // onShapeChange nor enqueue ever allocates or copies for them; build-phase objects, which may never run, wait
+    // for their first shape change as the reference does.
+    SkipLayerNormInterleavedPlugin(std::string const& name, bool mtron, Weights const& beta, Weights const& gamma,
+        bool onDevice)
         : BertPluginBase(name, kNAME, mtron ? "8" : "7", 2, mtron ? 2 : 1)
         , mMtron(mtron)
         , mLd(static_cast<int32_t>(beta.count))
@@ -259,12 +263,17 @@ public:
         TRTAMD_VALIDATE(beta.count == gamma.count);
         mBeta.assign(beta, DataType::kHALF);
         mGamma.assign(gamma, DataType::kHALF);
+        if (onDevice)
+        {
+            uploadParams();
+        }
     }
 
 protected:
     std::unique_ptr<BertPluginBase> doClone() override
     {
-        return std::make_unique<SkipLayerNormInterleavedPlugin>(mLayerName, mMtron, mBeta.view(), mGamma.view());
+        return std::make_unique<SkipLayerNormInterleavedPlugin>(mLayerName, mMtron, mBeta.view(), mGamma.view(),
+            mParamsOnDevice);
     }
 
     void doOutputTypes(DataType* outputTypes, DataType const* inputTypes) const override
@@ -298,13 +307,8 @@ protected:
         Dims const& d1 = in[1].dims;
         TRTAMD_VALIDATE(d0.nbDims == d1.nbDims);
         TRTAMD_VALIDATE(std::equal(d0.d, d0.d + d0.nbDims, d1.d));
-        // parameters go to the device on the first shape change, as in the reference
-        if (!mParamsOnDevice)
-        {
-            mGammaDev.upload(mGamma);
-            mBetaDev.upload(mBeta);
-            mParamsOnDevice = true;
-        }
+        // a build-phase object's parameters go to the device on its first shape change, as in the reference
+        uploadParams();
     }
 
     int32_t doEnqueue(PluginTensorDesc const* inputDesc, PluginTensorDesc const* outputDesc, void const* const* inputs,
@@ -355,6 +359,16 @@ protected:
     }
 
 private:
+    void uploadParams()
+    {
+        if (!mParamsOnDevice)
+        {
+            mGammaDev.upload(mGamma);
+            mBetaDev.upload(mBeta);
+            mParamsOnDevice = true;
+        }
+    }
+
     static void checkDescs(PluginTensorDesc const& iDesc, PluginTensorDesc const& sDesc, PluginTensorDesc const& oDesc)
     {
         TRTAMD_VALIDATE(iDesc.dims.nbDims == 4);
@@ -388,7 +402,8 @@ public:
     }
 
 protected:
-    std::unique_ptr<BertPluginBase> doCreate(char const* name, PluginFieldCollection const* fc, TensorRTPhase) override
+    std::unique_ptr<BertPluginBase> doCreate(char const* name, PluginFieldCollection const* fc,
+        TensorRTPhase phase) override
     {
         validateRequiredFields({"beta", "gamma"}, fc);
         Weights beta{DataType::kFLOAT, nullptr, 0};
@@ -399,7 +414,8 @@ protected:
         TRTAMD_VALIDATE_MSG(beta.count > 0, "SkipLayerNorm: invalid beta");
         TRTAMD_VALIDATE_MSG(gamma.values != nullptr, "SkipLayerNorm: invalid gamma");
         TRTAMD_VALIDATE_MSG(gamma.count > 0, "SkipLayerNorm: invalid gamma");
-        return std::make_unique<SkipLayerNormInterleavedPlugin>(name, mMtron, beta, gamma);
+        return std::make_unique<SkipLayerNormInterleavedPlugin>(name, mMtron, beta, gamma,
+            phase == TensorRTPhase::kRUNTIME);
     }
 
 private:

@@ -1,7 +1,8 @@
 // Native runner of a built INT8 BERT encoder (include/trtamd_encoder_runtime.h): what a deserialised engine
 // holds (runtime-phase plugin objects from the registry, device weights, activation scales) and the
-// stream-ordered sequence of plugin enqueues and linear layers that executes it.  enqueue() only launches:
-// every device allocation happens in set_embedding / set_layer, the activations live in the caller's workspace.
+// stream-ordered sequence of plugin enqueues and linear layers that executes it.  enqueue() only launches, the
+// first call included: every device allocation, copy and kernel attribute happens in set_embedding / set_layer
+// (which run each plugin's first shape change), the activations live in the caller's workspace.
 #include "plugin_common.h"
 #include "trtamd_encoder_runtime.h"
 
@@ -176,6 +177,23 @@ public:
         };
         L.ln1 = ln("_ln1", l.ln1_gamma, l.ln1_beta);
         L.ln2 = ln("_ln2", l.ln2_gamma, l.ln2_beta);
+        // One shape change with representative descriptors here, so that whatever a plugin sets up on its first
+        // shape change (device copies of parameters, kernel attributes) is done before the first enqueue, which
+        // a caller may be recording into a graph.
+        {
+            int64_t const T = mCfg.max_seqlen;
+            auto const il = TensorFormat::kCHW32;
+            auto const lin = TensorFormat::kLINEAR;
+            PluginTensorDesc const act = desc({1, E, T, 1}, DataType::kINT8, il, 1.f);
+            PluginTensorDesc const lnIn[2] = {act, act};
+            for (PluginPtr const* p : {&L.ln1, &L.ln2})
+            {
+                TRTAMD_VALIDATE_MSG(runtimeOf(*p)->onShapeChange(lnIn, 2, &act, 1) == 0, tag + ": SkipLayerNorm set-up failed");
+            }
+            PluginTensorDesc const qIn[3] = {desc({1, 3 * E, T, 1}, DataType::kINT8, il, 1.f),
+                desc({2}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f)};
+            TRTAMD_VALIDATE_MSG(runtimeOf(L.attention)->onShapeChange(qIn, 3, &act, 1) == 0, tag + ": attention set-up failed");
+        }
         L.sX = l.s_x;
         L.sQkv = l.s_qkv;
         L.sCtx = l.s_ctx;

@@ -397,16 +397,27 @@ class Int8BertEncoder:
             self.build_native()
         if ids is not None:
             self._bind(ids, segs, cu)
-        torch, api, b = self.torch, self.api, self.buf
-        need = api.encoder_workspace_size(self._native, self.T)
-        if self._native_ws is None or self._native_ws.numel() < need:
-            self._native_ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
-        if "out_native" not in b or b["out_native"].shape[0] != self.T:
-            b["out_native"] = torch.empty((self.T, self.cfg.hidden), dtype=torch.float16, device="cuda")
+        api, b = self.api, self.buf
+        self.prepare_native()
         api.check(api.encoder_enqueue(self._native, b["ids"].data_ptr(), b["segs"].data_ptr(), b["cu"].data_ptr(), self.B,
                                       self.T, self._native_ws.data_ptr(), b["out_native"].data_ptr(),
                                       self.stream if stream is None else stream))
         return b["out_native"]
+
+    def prepare_native(self):
+        """The caller's side of an enqueue that must not allocate: workspace and output tensor for the bound batch."""
+        torch, b = self.torch, self.buf
+        need = self.api.encoder_workspace_size(self._native, self.T)
+        if self._native_ws is None or self._native_ws.numel() < need:
+            self._native_ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
+        if "out_native" not in b or b["out_native"].shape[0] != self.T:
+            b["out_native"] = torch.empty((self.T, self.cfg.hidden), dtype=torch.float16, device="cuda")
+
+    def destroy_native(self):
+        h = getattr(self, "_native", None)
+        if h:
+            self.api.encoder_destroy(h)
+            self._native = None
 
     def __del__(self):
         h = getattr(self, "_native", None)

@@ -109,3 +109,76 @@ def f32_bits(x):
 def half2_bits(x):
     h = int(np.float16(x).view(np.uint16))
     return h | (h << 16)
+
+
+# ---- INT8 fused attention on cu_seqlens: the strict decomposition used wherever that kernel is checked ----
+
+def int8_attention_parity(qkv, cu, N, s1, ss, s2, interleaved, S=None, expect=None, D=64):
+    """Runs the shipped INT8 var-seqlen kernel and the instantiation that dumps its intermediates on qkv
+    ([T, 3*N*D] int8, channel order [N][3][D]) and checks, against the oracle:
+    both give the same bytes (and `expect`, [T, N*D], if given); first-GEMM accumulators bit-exact; quantised
+    probabilities within 1 with at most max(2, 1e-5 n) off; the second GEMM and the requantisation exact from the
+    kernel's own probabilities; rows whose probabilities all agree equal the oracle's bit for bit.
+    Returns the kernel's output [T, N*D]."""
+    import ctypes as C
+
+    import oracle
+    from tensorrt_amd import capi
+    api = capi.api()
+    cu = np.asarray(cu, np.int32)
+    lens = np.diff(cu)
+    B, T = len(lens), int(cu[-1])
+    S = int(S or max(int(lens.max()), 1))
+    ref, a1, p8, _ = oracle.mha_fused_i8_packed(qkv, cu, N, D, s1, ss, s2, want_ints=True)
+    if interleaved:
+        x = qkv.reshape(T, N, 3, D).transpose(0, 2, 1, 3).reshape(T, 3 * N * D)
+        d_qkv = dev(oracle.interleave(x))
+    else:
+        d_qkv = dev(qkv)
+    d_dbg = dev_empty((T * N * D,), np.int8, fill=0x55)
+    d_out = dev_empty((T * N * D,), np.int8, fill=0x55)
+    d_cu = dev(cu)
+    d_a1 = dev_empty((B, N, S, S), np.int32, fill=0)
+    d_p8 = dev_empty((B, N, S, S), np.int8, fill=0)
+    p = capi.FmhaParams()
+    p.qkv_ptr, p.o_ptr, p.cu_seqlens = ptr(d_qkv), ptr(d_dbg), ptr(d_cu)
+    p.b, p.h, p.s, p.d = B, N, S, D
+    p.scale_bmm1, p.scale_softmax, p.scale_bmm2 = f32_bits(s1), f32_bits(ss), f32_bits(s2)
+    p.interleaved, p.use_int8_scale_max = int(interleaved), 1
+    p.qkv_stride_in_bytes = T if interleaved else 3 * N * D
+    p.o_stride_in_bytes = T if interleaved else N * D
+    api.check(api.fused_mha_run_debug(stream(), 2, C.byref(p), ptr(d_a1), ptr(d_p8)))
+    p.o_ptr = ptr(d_out)
+    api.check(api.fused_mha_run(stream(), 2, C.byref(p)))
+    sync()
+    got = host(d_out)
+    # the shipped instantiation must give the same bytes as the checked one, fill pattern of unowned rows included
+    assert np.array_equal(got, host(d_dbg)), "shipped INT8 kernel differs from the instantiation that dumps intermediates"
+    got = oracle.deinterleave(got, T, N * D) if interleaved else got.reshape(T, N * D)
+    if expect is not None:
+        assert np.array_equal(got, np.asarray(expect).reshape(T, N * D)), "kernel output differs from the tensor under test"
+    g_a1, g_p8 = host(d_a1), host(d_p8)
+    ref3, got3 = ref.reshape(T, N, D), got.reshape(T, N, D)
+    n_p8 = n_off = 0
+    for b in range(B):
+        L = int(lens[b])
+        if L == 0:
+            continue
+        lo, hi = int(cu[b]), int(cu[b + 1])
+        assert np.array_equal(g_a1[b, :, :L, :L], a1[b, :, :L, :L]), "first-GEMM accumulators must be bit-exact"
+        dp = g_p8[b, :, :L, :L].astype(np.int32) - p8[b, :, :L, :L]
+        assert np.abs(dp).max() <= 1, "quantised probabilities differ by more than 1 LSB"
+        n_p8 += dp.size
+        n_off += int((dp != 0).sum())
+        # exact second GEMM from the kernel's own p8
+        v = qkv[lo:hi].reshape(L, N, 3, D)[:, :, 2, :].astype(np.int64)               # [L,N,D]
+        acc2 = np.einsum("nqk,knd->qnd", g_p8[b, :, :L, :L].astype(np.int64), v)        # [L,N,D]
+        want = np.clip(np.rint(acc2.astype(np.float32) * np.float32(s2)), -128, 127).astype(np.int8)
+        assert np.array_equal(got3[lo:hi], want), "second GEMM / requantisation must be exact"
+        # (query, head) rows whose probabilities agree with the oracle agree with it bit for bit; a probability
+        # that rounds the other way (exp differs in the last ulp) moves 64 outputs by up to |v| * scale_bmm2,
+        # which the exact check above already covers.
+        same = (dp == 0).all(axis=2).T                                                  # [L(q), N]
+        assert np.array_equal(got3[lo:hi][same], ref3[lo:hi][same])
+    assert n_off <= max(2, 1e-5 * n_p8), f"{n_off} of {n_p8} probabilities differ from the oracle"
+    return got

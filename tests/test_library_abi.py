@@ -36,6 +36,26 @@ def test_kernel_header_symbols_exported(lib):
     assert sorted(capi.HEADER_SYMBOLS) == names
 
 
+def test_test_hook_header_symbols_exported(lib):
+    names = _declared("trtamd_test_hooks.h", "TRTAMD_API")
+    assert names == sorted(capi.TEST_HOOK_SYMBOLS)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in trtamd_test_hooks.h but not exported"
+
+
+def test_every_exported_trtamd_symbol_is_declared_in_a_header(lib):
+    """Nothing is exported behind the headers' back."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", tensorrt_amd._LIB], capture_output=True, text=True, check=True)
+    exported = {l.split()[-1] for l in out.stdout.splitlines() if " T " in l and l.split()[-1].startswith("trtamd_")}
+    declared = set()
+    for h, macro in (("trtamd_bert_kernels.h", "TRTAMD_API"), ("trtamd_test_hooks.h", "TRTAMD_API"),
+                     ("trtamd_encoder_ops.h", "TRTAMD_API"), ("trtamd_encoder_runtime.h", "TRTAMD_API"),
+                     ("trtamd_plugin_c.h", "TRTAMD_PLUGIN_API")):
+        declared |= set(_declared(h, macro))
+    assert exported <= declared, sorted(exported - declared)
+
+
 def test_encoder_ops_header_symbols_exported(lib):
     names = _declared("trtamd_encoder_ops.h", "TRTAMD_API")
     assert names
