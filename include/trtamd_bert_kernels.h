@@ -153,6 +153,17 @@ TRTAMD_API size_t trtamd_unfused_mha_workspace_size(int32_t type, int32_t S, int
 TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
     void const* qkv, int32_t const* maskIdx, void* output, void* workspace);
 
+/* trtamd_unfused_mha for callers that cannot allocate (code under graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference: the score matrices live in a device array that belongs to
+ * the library (trtamd_unfused_mha_static_capacity() bytes, 32 MiB, held by every GPU the library runs on until the
+ * process ends) instead of a caller workspace.  Neither call allocates, frees or synchronises; the first call on a
+ * device looks the array's address up.  A problem whose trtamd_unfused_mha_workspace_size exceeds the capacity is
+ * refused with TRTAMD_STATUS_NOT_SUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU
+ * (different streams) race; calls on one stream, or ordered by events, are safe. */
+TRTAMD_API size_t trtamd_unfused_mha_static_capacity(void);
+TRTAMD_API int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N,
+    int32_t d, void const* qkv, int32_t const* maskIdx, void* output);
+
 /* Parameter block of the fused kernels: the fields of Fused_multihead_attention_params_v2
  * (plugin/bertQKVToContextPlugin/fused_multihead_attention_v2/fused_multihead_attention_v2.h:31-101)
  * and Fused_multihead_attention_params

@@ -100,6 +100,8 @@ _SIGS = {
     "trtamd_scaled_softmax_fp16": (C.c_int, [c_p, i32, i32, i32, f32, c_p, c_p, c_p]),
     "trtamd_unfused_mha_workspace_size": (C.c_size_t, [i32, i32, i32, i32]),
     "trtamd_unfused_mha": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p, c_p]),
+    "trtamd_unfused_mha_static_capacity": (C.c_size_t, []),
+    "trtamd_unfused_mha_static": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p]),
     "trtamd_fused_mha_run": (C.c_int, [c_p, i32, C.POINTER(FmhaParams)]),
     "trtamd_fused_mha_run_debug": (C.c_int, [c_p, i32, C.POINTER(FmhaParams), c_p, c_p]),
     "trtamd_fused_mha_prepare": (C.c_int, []),

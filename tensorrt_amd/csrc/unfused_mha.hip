@@ -9,11 +9,51 @@
 #include "host_utils.hpp"
 
 #include <algorithm>
+#include <mutex>
+
+// Score matrices of trtamd_unfused_mha_static: device memory that belongs to the library instead of the caller.
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.  In
+// host code the name below is only a stand-in for the symbol (it is not a device address): host code goes through
+// the per-device pointer that static_scratch() obtains with hipGetSymbolAddress.
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace trtamd
 {
 namespace
 {
+
+constexpr int kMaxDevices = 64;
+
+// Device address of `scratch` on the current device, looked up once per device (with that device current).
+int static_scratch(void** out)
+{
+    static std::mutex mtx;
+    static void* ptrs[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    {
+        (void) hipGetLastError();
+        return set_error(TRTAMD_STATUS_FAILURE, "unfused MHA (static scratch): no current device (%s)",
+            hipGetErrorString(e));
+    }
+    std::lock_guard<std::mutex> lock(mtx);
+    if (ptrs[dev] == nullptr)
+    {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+        {
+            (void) hipGetLastError();
+            return set_error(TRTAMD_STATUS_FAILURE, "unfused MHA (static scratch): hipGetSymbolAddress failed on device %d: %s",
+                dev, hipGetErrorString(e));
+        }
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return TRTAMD_STATUS_SUCCESS;
+}
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWaveSize;
@@ -337,6 +377,42 @@ extern "C" int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
     }
     return unfused_mha<f16>(as_stream(stream), S, B, N, d, static_cast<f16 const*>(qkv), maskIdx,
         static_cast<f16*>(output), workspace);
+}
+
+extern "C" size_t trtamd_unfused_mha_static_capacity(void)
+{
+    return kStaticScratchBytes;
+}
+
+extern "C" int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
+    void const* qkv, int32_t const* maskIdx, void* output)
+{
+    if (type != 0 && type != 1)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: data type %d (only FP32=0 and FP16=1)", type);
+    }
+    if (S <= 0 || B <= 0 || N <= 0 || d <= 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
+    }
+    // 2 * wordSize * S*S * B*N in 128-bit arithmetic free of overflow: each factor is below 2^31
+    double const need = 2.0 * (type == 0 ? 4.0 : 2.0) * (double) S * (double) S * (double) B * (double) N;
+    if (need > (double) kStaticScratchBytes)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED,
+            "unfused MHA (static scratch): S=%d B=%d N=%d needs %.0f bytes of score matrices, the library's array holds "
+            "%zu; use trtamd_unfused_mha with a workspace",
+            S, B, N, need, kStaticScratchBytes);
+    }
+    void* ws = nullptr;
+    int const st = static_scratch(&ws);
+    if (st != TRTAMD_STATUS_SUCCESS)
+    {
+        return st;
+    }
+    // every score the second and third kernel read was written by the kernel before it in this call: nothing in
+    // the array has to start at zero, and what the previous call left there is never read
+    return trtamd_unfused_mha(stream, type, S, B, N, d, qkv, maskIdx, output, ws);
 }
 
 extern "C" int trtamd_zero_padding_2d(
