@@ -17,6 +17,7 @@ CSRC = os.path.join(ROOT, "csrc")
 INCLUDE = os.path.join(os.path.dirname(ROOT), "include")
 LIB_DIR = os.path.join(ROOT, "lib")
 LIB_NAME = "libtrtamd_bert_plugins.so"
+MICROBENCH_LIB_NAME = "libtrtamd_microbench.so"   # instruction-rate probes for bench.py; not part of the plugin library
 OBJ_DIR = os.path.join(CSRC, "_obj")
 
 ARCH = "gfx950"
@@ -76,5 +77,23 @@ def build_library(jobs: int | None = None, verbose: bool = False) -> str:
     return out
 
 
+def build_microbench(verbose: bool = False) -> str:
+    """The instruction-rate microbenchmarks (csrc/bench/microbench.hip) as a library of their own."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(CSRC, "bench", "microbench.hip")
+    out = os.path.join(LIB_DIR, MICROBENCH_LIB_NAME)
+    tmp = out + ".tmp"
+    cmd = [_hipcc(), *COMMON_FLAGS, "-x", "hip", "-shared", src, "-o", tmp]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    os.replace(tmp, out)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build_library(verbose=True)
+    build_microbench(verbose=True)

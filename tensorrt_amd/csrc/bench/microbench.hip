@@ -1,0 +1,292 @@
+// On-box instruction-rate microbenchmarks for gfx950 (libtrtamd_microbench.so, loaded by bench.py only): what the
+// matrix and vector pipes of this GPU sustain for the instructions the attention and linear kernels are made of.
+// Every kernel runs register-only loops of independent chains on every SIMD of the chip; the host function times
+// a few launches with events and returns milliseconds per launch.  Not part of the plugin library.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+namespace
+{
+
+constexpr int kThreads = 256; // 4 wavefronts: one per SIMD of a CU
+
+// A and B operands of one lane: zeros, or bytes from a buffer of random data (so the values cannot be folded)
+__device__ inline i32x4 operand(int32_t const* src, int which)
+{
+    i32x4 v;
+    for (int i = 0; i < 4; ++i)
+    {
+        v[i] = src[(which * 64 + (threadIdx.x & 63)) * 4 + i];
+    }
+    return v;
+}
+
+// CHAINS independent accumulators per wavefront, each updated once per iteration
+template <int CHAINS>
+__global__ __launch_bounds__(kThreads) void mfma_16x16x64_i8_kernel(int32_t const* src, int32_t* out, int iters)
+{
+    i32x4 const a = operand(src, 0), b = operand(src, 1);
+    i32x4 acc[CHAINS];
+    for (int c = 0; c < CHAINS; ++c)
+    {
+        acc[c] = i32x4{c, 0, 0, 0};
+    }
+    for (int it = 0; it < iters; ++it)
+    {
+        // inline assembly pins each accumulator to its own vector registers: left to the compiler, four or more
+        // chains in a loop are shuffled through the accumulation registers with a dozen copies per iteration
+#pragma unroll
+        for (int c = 0; c < CHAINS; ++c)
+        {
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[c]) : "v"(a), "v"(b));
+        }
+    }
+    int s = 0;
+    for (int c = 0; c < CHAINS; ++c)
+    {
+        s += acc[c][0] + acc[c][1] + acc[c][2] + acc[c][3];
+    }
+    out[blockIdx.x * kThreads + threadIdx.x] = s;
+}
+
+template <int CHAINS>
+__global__ __launch_bounds__(kThreads) void mfma_32x32x32_i8_kernel(int32_t const* src, int32_t* out, int iters)
+{
+    i32x4 const a = operand(src, 0), b = operand(src, 1);
+    i32x16 acc[CHAINS];
+    for (int c = 0; c < CHAINS; ++c)
+    {
+        for (int i = 0; i < 16; ++i)
+        {
+            acc[c][i] = c + i;
+        }
+    }
+    for (int it = 0; it < iters; ++it)
+    {
+#pragma unroll
+        for (int c = 0; c < CHAINS; ++c)
+        {
+            asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc[c]) : "v"(a), "v"(b));
+        }
+    }
+    int s = 0;
+    for (int c = 0; c < CHAINS; ++c)
+    {
+        for (int i = 0; i < 16; ++i)
+        {
+            s += acc[c][i];
+        }
+    }
+    out[blockIdx.x * kThreads + threadIdx.x] = s;
+}
+
+// Eight independent chains of one vector-ALU instruction
+enum ValuOp
+{
+    OP_FMA = 0,
+    OP_EXP = 1,
+    OP_ADD = 2,
+    OP_PERM = 3,
+    OP_MAX3 = 4,
+    OP_CVT_PK_U8 = 5,
+    OP_SOFTMAX_MIX = 6, // fma, exp, add, fma per element: the inner sequence of the attention kernel
+};
+
+template <int OP>
+__global__ __launch_bounds__(kThreads) void valu_kernel(int32_t const* src, int32_t* out, int iters, int64_t* clocks)
+{
+    uint64_t const c0 = __builtin_readcyclecounter();
+    uint64_t const w0 = wall_clock64();
+    float const c = __int_as_float(src[0] & 0x007fffff | 0x3f800000) * 0.5f + 0.25f; // in [0.75, 1.25)
+    float a[8];
+    float sum = 0.f;
+    for (int i = 0; i < 8; ++i)
+    {
+        a[i] = (float) (threadIdx.x & 63) * 0.001f + (float) i;
+    }
+    for (int it = 0; it < iters; ++it)
+    {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+        {
+            if (OP == OP_FMA)
+            {
+                a[i] = __builtin_fmaf(a[i], c, 0.5f);
+            }
+            else if (OP == OP_EXP)
+            {
+                a[i] = __builtin_amdgcn_exp2f(a[i]);
+            }
+            else if (OP == OP_ADD)
+            {
+                a[i] = a[i] + c;
+            }
+            else if (OP == OP_PERM)
+            {
+                a[i] = __uint_as_float(__builtin_amdgcn_perm(__float_as_uint(a[i]), __float_as_uint(a[(i + 1) & 7]),
+                    0x05040100u));
+            }
+            else if (OP == OP_MAX3)
+            {
+                a[i] = __int_as_float(max(max(__float_as_int(a[i]), __float_as_int(a[(i + 1) & 7])),
+                    __float_as_int(a[(i + 2) & 7])));
+            }
+            else if (OP == OP_CVT_PK_U8)
+            {
+                a[i] = __uint_as_float(__builtin_amdgcn_cvt_pk_u8_f32(a[i], 1, __float_as_uint(a[(i + 1) & 7])));
+            }
+            else
+            {
+                float const e = __builtin_amdgcn_exp2f(__builtin_fmaf(a[i], c, -1.0f));
+                sum += e;
+                a[i] = __builtin_fmaf(e, c, 12582912.f);
+            }
+        }
+    }
+    float s = sum;
+    for (int i = 0; i < 8; ++i)
+    {
+        s += a[i];
+    }
+    out[blockIdx.x * kThreads + threadIdx.x] = __float_as_int(s);
+    if (clocks && threadIdx.x == 0)
+    {
+        // shader-clock cycles and 100 MHz wall-clock ticks this workgroup's first wavefront spent in the loop
+        clocks[2 * blockIdx.x] = (int64_t) (__builtin_readcyclecounter() - c0);
+        clocks[2 * blockIdx.x + 1] = (int64_t) (wall_clock64() - w0);
+    }
+}
+
+// One MFMA and NV independent vector-ALU instructions per step, in one wavefront's instruction stream: does the
+// matrix pipe run beside the vector ALU (time = max of the two) or in its place (time = sum)?
+template <int NV>
+__global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* src, int32_t* out, int iters)
+{
+    i32x4 const a = operand(src, 0), b = operand(src, 1);
+    float const c = __int_as_float(src[0] & 0x007fffff | 0x3f800000) * 0.5f + 0.25f;
+    i32x4 acc[4];
+    float f[8];
+    for (int i = 0; i < 4; ++i)
+    {
+        acc[i] = i32x4{i, 0, 0, 0};
+    }
+    for (int i = 0; i < 8; ++i)
+    {
+        f[i] = (float) (threadIdx.x & 63) * 0.001f + (float) i;
+    }
+    for (int it = 0; it < iters; ++it)
+    {
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+        {
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a), "v"(b));
+#pragma unroll
+            for (int v = 0; v < NV; ++v)
+            {
+                asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(f[(m * NV + v) & 7]) : "v"(c));
+            }
+        }
+    }
+    int s = 0;
+    for (int i = 0; i < 4; ++i)
+    {
+        s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    }
+    float t = 0.f;
+    for (int i = 0; i < 8; ++i)
+    {
+        t += f[i];
+    }
+    out[blockIdx.x * kThreads + threadIdx.x] = s + __float_as_int(t);
+}
+
+template <typename Launch>
+float time_launches(Launch launch, int reps)
+{
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+    {
+        return -1.f;
+    }
+    launch();
+    launch();
+    (void) hipDeviceSynchronize();
+    (void) hipEventRecord(e0, nullptr);
+    for (int i = 0; i < reps; ++i)
+    {
+        launch();
+    }
+    (void) hipEventRecord(e1, nullptr);
+    (void) hipEventSynchronize(e1);
+    float ms = -1.f;
+    (void) hipEventElapsedTime(&ms, e0, e1);
+    (void) hipEventDestroy(e0);
+    (void) hipEventDestroy(e1);
+    return hipGetLastError() == hipSuccess ? ms / (float) reps : -1.f;
+}
+
+} // namespace
+
+#define MB_API extern "C" __attribute__((visibility("default")))
+
+// Milliseconds per launch of `blocks` workgroups of 4 wavefronts, each wavefront issuing iters * chains MFMAs.
+// shape: 0 = v_mfma_i32_16x16x64_i8, 1 = v_mfma_i32_32x32x32_i8 (both 32768 integer operations per instruction
+// and wavefront); chains: 1, 2, 4 or 8 independent accumulators; operands: 128 x 4 int32 of device memory.
+MB_API float trtamd_microbench_mfma_i8(int shape, int chains, int blocks, int iters, int32_t const* operands, int32_t* out)
+{
+#define MB_CASE(S, C)                                                                                                  \
+    if (shape == S && chains == C)                                                                                     \
+    {                                                                                                                  \
+        return time_launches(                                                                                          \
+            [&] {                                                                                                      \
+                if (S == 0)                                                                                            \
+                    hipLaunchKernelGGL((mfma_16x16x64_i8_kernel<C>), dim3(blocks), dim3(kThreads), 0, nullptr,         \
+                        operands, out, iters);                                                                         \
+                else                                                                                                   \
+                    hipLaunchKernelGGL((mfma_32x32x32_i8_kernel<C>), dim3(blocks), dim3(kThreads), 0, nullptr,         \
+                        operands, out, iters);                                                                         \
+            },                                                                                                         \
+            5);                                                                                                        \
+    }
+    MB_CASE(0, 1) MB_CASE(0, 2) MB_CASE(0, 4) MB_CASE(0, 8) MB_CASE(1, 1) MB_CASE(1, 2) MB_CASE(1, 4) MB_CASE(1, 8)
+#undef MB_CASE
+    return -1.f;
+}
+
+// Milliseconds per launch; every wavefront issues iters * 4 steps of (one v_mfma_i32_16x16x64_i8, nv v_fma_f32).
+MB_API float trtamd_microbench_mfma_valu(int nv, int blocks, int iters, int32_t const* operands, int32_t* out)
+{
+#define MB_NV(V)                                                                                                       \
+    if (nv == V)                                                                                                       \
+    {                                                                                                                  \
+        return time_launches(                                                                                          \
+            [&] {                                                                                                      \
+                hipLaunchKernelGGL((mfma_valu_mix_kernel<V>), dim3(blocks), dim3(kThreads), 0, nullptr, operands, out, \
+                    iters);                                                                                            \
+            },                                                                                                         \
+            5);                                                                                                        \
+    }
+    MB_NV(0) MB_NV(1) MB_NV(2) MB_NV(3) MB_NV(4) MB_NV(6) MB_NV(8) MB_NV(12)
+#undef MB_NV
+    return -1.f;
+}
+
+// Milliseconds per launch; every wavefront issues iters * 8 instructions of kind `op` (ValuOp; OP_SOFTMAX_MIX
+// issues iters * 8 groups of four).
+// clocks (optional): 2 x blocks int64, per workgroup the shader-clock cycles and the 100 MHz ticks of its loop.
+MB_API float trtamd_microbench_valu(int op, int blocks, int iters, int32_t const* operands, int32_t* out, int64_t* clocks)
+{
+#define MB_OP(O)                                                                                                       \
+    if (op == O)                                                                                                       \
+    {                                                                                                                  \
+        return time_launches(                                                                                          \
+            [&] { hipLaunchKernelGGL((valu_kernel<O>), dim3(blocks), dim3(kThreads), 0, nullptr, operands, out, iters, clocks); }, \
+            5);                                                                                                        \
+    }
+    MB_OP(OP_FMA) MB_OP(OP_EXP) MB_OP(OP_ADD) MB_OP(OP_PERM) MB_OP(OP_MAX3) MB_OP(OP_CVT_PK_U8) MB_OP(OP_SOFTMAX_MIX)
+#undef MB_OP
+    return -1.f;
+}

@@ -254,4 +254,27 @@ __device__ inline uint32_t xcd_remap(uint32_t bid, uint32_t nblocks)
     return (bid % kXcds) * per + bid / kXcds;
 }
 
+// 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane i's bytes land at LDS byte
+// address ldsAddr + 16 i, so one instruction of a wavefront fills 1 KB; ldsAddr is wave-uniform and travels in M0.
+// The data never passes through vector registers, and completion is counted by vmcnt like any vector-memory load.
+// Written as inline assembly on purpose: the compiler then neither counts these loads nor orders LDS reads behind
+// them, and the kernel below places its own s_waitcnt where a stage must have landed.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm" // M0 is named as clobbered on purpose
+__device__ __forceinline__ void load_to_lds16(void const* g, uint32_t ldsAddr)
+{
+    // readfirstlane: a value the compiler cannot prove wave-uniform would otherwise arrive in a vector register
+    uint32_t const uniform = (uint32_t) __builtin_amdgcn_readfirstlane((int) ldsAddr);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(uniform) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+// s_waitcnt vmcnt(N) alone (the other counters at their maxima): gfx9 encoding, vmcnt in bits 3:0 and 15:14
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
 } // namespace trtamd

@@ -755,18 +755,18 @@ __device__ inline void stage_kv_prefix_i8(FmhaArgs const& a, int64_t seqBase, in
     }
 }
 
-// All query tiles of this wavefront for a sequence of exactly NKB key blocks (the last one ragged).
+// One 16-query tile of a sequence of exactly NKB key blocks (the last one ragged): query tile qt of the sequence sq,
+// head n; qreg = the tile's Q^T operand (16 bytes d = 16g .. 16g+15 of query 16 qt + lane % 16, zero beyond the
+// sequence).  sK / sV: the head's keys and values in LDS as stage_kv_prefix_i8 lays them out.
 template <int NKB, bool INTERLEAVED, bool DEBUG>
-__device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, int const b, int const n,
-    int const qtBegin, int const qtEnd, uint8_t const* sK, uint8_t const* sV, i32x4 const qFirst)
+__device__ __forceinline__ void tile_i8(FmhaArgs const& a, SeqInfo const& sq, int const b, int const n, int const qt,
+    uint8_t const* sK, uint8_t const* sV, i32x4 const qreg)
 {
     constexpr int kRow = Lds<1>::kRow;
     constexpr int NT = NKB * 4;
     int const lane = threadIdx.x & (kWaveSize - 1);
-    int const wave = threadIdx.x >> 6;
     int const lq = lane & 15;
     int const g = lane >> 4;
-    uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
 
     // last block: keys 64(NKB-1) + 16u + 4g + j exist for (16u + 4g + j) < lastKeys
     int const lastKeys = sq.nk - (NKB - 1) * 64;
@@ -774,203 +774,217 @@ __device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, 
     i32x4 const seedFull = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
     int const lastRel = lastKeys - 4 * g; // key 16u + j of this lane group exists iff 16u + j < lastRel
 
-    auto load_q = [&](int qt) -> i32x4 {
-        int const qq = qt * kQPerWave + lq;
-        i32x4 v = {0, 0, 0, 0};
-        if (qq < sq.nq)
-        {
-            v = *reinterpret_cast<i32x4 const*>(
-                src + qkv_chunk_offset<1, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, g));
-        }
-        return v;
-    };
-    constexpr int qtStep = kWavesI8;
-    i32x4 qnext = qFirst; // requested by the caller together with K and V
-    for (int qt = qtBegin + wave; qt < qtEnd; qt += qtStep)
+    int const q = qt * kQPerWave + lq;
+    bool const qValid = q < sq.nq;
+
+    // ---- S^T = K Q^T; the int32 result reads as binary32 12582912 + acc, -inf for absent keys
+    i32x4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
     {
-        int const q = qt * kQPerWave + lq;
-        bool const qValid = q < sq.nq;
-        i32x4 const qreg = qnext;
-        qnext = load_q(qt + qtStep);
-
-        // ---- S^T = K Q^T; the int32 result reads as binary32 12582912 + acc, -inf for absent keys
-        i32x4 acc[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
+        int const key = t * 16 + lq;
+        i32x4 const kreg = *reinterpret_cast<i32x4 const*>(sK + key * kRow + swz<1>(key, g) * 16);
+        i32x4 seed = seedFull;
+        if (t >= NT - 4)
         {
-            int const key = t * 16 + lq;
-            i32x4 const kreg = *reinterpret_cast<i32x4 const*>(sK + key * kRow + swz<1>(key, g) * 16);
-            i32x4 seed = seedFull;
-            if (t >= NT - 4)
-            {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    seed[j] = (16 * (t & 3) + j) < lastRel ? kMagicBits : kNegInfBits;
-                }
-            }
-            acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kreg, qreg, seed, 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-
-        if (DEBUG && a.dbgAcc1 && qValid)
-        {
-            for (int t = 0; t < NT; ++t)
-            {
-                for (int j = 0; j < 4; ++j)
-                {
-                    int const key = t * 16 + g * 4 + j;
-                    if (key < sq.nk)
-                    {
-                        a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key] = acc[t][j] - kMagicBits;
-                    }
-                }
-            }
-        }
-
-        // ---- row max on the biased integers (monotone in the score; -inf is a negative pattern)
-        // two chains of three-input maxima (v_max3_i32): one instruction per two scores
-        int mxA = kNegInfBits, mxB = kNegInfBits;
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-        {
-            mxA = max(max(mxA, acc[t][0]), acc[t][1]);
-            mxB = max(max(mxB, acc[t][2]), acc[t][3]);
-        }
-        int mx = max(mxA, mxB);
-        mx = reduce_step<16>(mx, [](int x, int y) { return max(x, y); });
-        mx = reduce_step<32>(mx, [](int x, int y) { return max(x, y); });
-        __builtin_amdgcn_sched_barrier(0);
-
-        // ---- e = 2^((acc - max) * c) in place, row sum
-        float const negK0 = -__int_as_float(mx) * a.c;
-        float sum0 = 0.f, sum1 = 0.f;
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-        {
-            if ((t & 3) == 0)
-            {
-                __builtin_amdgcn_sched_barrier(0); // bound the live temporaries to one key block
-            }
-            if (t >= NT - 4 && (t & 3) >= lastTiles)
-            {
-                continue; // tile without keys: its accumulators keep the -inf pattern (p8 = 0 below)
-            }
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
-                float const ev = __builtin_amdgcn_exp2f(fmaf(__int_as_float(acc[t][j]), a.c, negK0));
-                acc[t][j] = __float_as_int(ev);
-                if (j & 1)
-                {
-                    sum1 += ev;
-                }
-                else
-                {
-                    sum0 += ev;
-                }
+                seed[j] = (16 * (t & 3) + j) < lastRel ? kMagicBits : kNegInfBits;
             }
         }
-        float sum = sum0 + sum1;
-        sum = reduce_step<16>(sum, [](float x, float y) { return x + y; });
-        sum = reduce_step<32>(sum, [](float x, float y) { return x + y; });
-        float const r = a.scaleSoftmax / sum;   // sum >= 1: the row maximum contributes 2^0
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kreg, qreg, seed, 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
-        // ---- p8 = rne(e * r), four keys to a dword; O^T = V^T P^T
-        i32x4 oacc[4];
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+    if (DEBUG && a.dbgAcc1 && qValid)
+    {
+        for (int t = 0; t < NT; ++t)
         {
-            oacc[dt] = i32x4{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-        {
-            __builtin_amdgcn_sched_barrier(0);
-            i32x4 preg = {0, 0, 0, 0};
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int j = 0; j < 4; ++j)
             {
-                if (kb == NKB - 1 && u >= lastTiles)
+                int const key = t * 16 + g * 4 + j;
+                if (key < sq.nk)
                 {
-                    continue;
+                    a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key] = acc[t][j] - kMagicBits;
                 }
-                uint32_t yb[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    yb[j] = __float_as_uint(fmaf(__int_as_float(acc[kb * 4 + u][j]), r, kMagic));
-                }
-                uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
-                uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-                preg[u] = (int) __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-            }
-            if (DEBUG && a.dbgP8 && qValid)
-            {
-                for (int u = 0; u < 4; ++u)
-                {
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        int const key = kb * 64 + u * 16 + g * 4 + j;
-                        if (key < sq.nk)
-                        {
-                            a.dbgP8[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
-                                = (int8_t) ((uint32_t) preg[u] >> (8 * j));
-                        }
-                    }
-                }
-            }
-            int const vrow = kb * 64 + 8 * g + (lq >> 1);
-            uint8_t const* vbase = sV + vrow * kRow + 8 * (lq & 1);
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-            {
-                int const sc = swz<1>(vrow, dt) * 16;
-                i32x2 const v0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + sc));
-                i32x2 const v1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + 32 * kRow + sc));
-                i32x4 const vreg = {v0[0], v0[1], v1[0], v1[1]};
-                oacc[dt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vreg, preg, oacc[dt], 0, 0, 0);
             }
         }
+    }
 
-        // ---- out8 = sat8(rne(acc2 * scale_bmm2)): binary32 product (rounded on its own, not fused
-        //      into the add), rounded to an integer through the magic constant, clamped on the bit
-        //      patterns (monotone for the positive results; anything negative is below the range).
-        //      Lane (g, query) then holds bytes 4g..4g+3 of each 16-byte quarter dt of the query's row; a 4 x 4
-        //      transpose over the four rows of 16 lanes (v_permlane32_swap, v_permlane16_swap) leaves it with the
-        //      whole quarter dt = g, which goes out as one 16-byte store.
-        uint32_t pk[4];
+    // ---- row max on the biased integers (monotone in the score; -inf is a negative pattern)
+    // two chains of three-input maxima (v_max3_i32): one instruction per two scores
+    int mxA = kNegInfBits, mxB = kNegInfBits;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+    for (int t = 0; t < NT; ++t)
+    {
+        mxA = max(max(mxA, acc[t][0]), acc[t][1]);
+        mxB = max(max(mxB, acc[t][2]), acc[t][3]);
+    }
+    int mx = max(mxA, mxB);
+    mx = reduce_step<16>(mx, [](int x, int y) { return max(x, y); });
+    mx = reduce_step<32>(mx, [](int x, int y) { return max(x, y); });
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- e = 2^((acc - max) * c) in place, row sum
+    float const negK0 = -__int_as_float(mx) * a.c;
+    float sum0 = 0.f, sum1 = 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+    {
+        if ((t & 3) == 0)
         {
+            __builtin_amdgcn_sched_barrier(0); // bound the live temporaries to one key block
+        }
+        if (t >= NT - 4 && (t & 3) >= lastTiles)
+        {
+            continue; // tile without keys: its accumulators keep the -inf pattern (p8 = 0 below)
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            float const ev = __builtin_amdgcn_exp2f(fmaf(__int_as_float(acc[t][j]), a.c, negK0));
+            acc[t][j] = __float_as_int(ev);
+            if (j & 1)
+            {
+                sum1 += ev;
+            }
+            else
+            {
+                sum0 += ev;
+            }
+        }
+    }
+    float sum = sum0 + sum1;
+    sum = reduce_step<16>(sum, [](float x, float y) { return x + y; });
+    sum = reduce_step<32>(sum, [](float x, float y) { return x + y; });
+    float const r = a.scaleSoftmax / sum;   // sum >= 1: the row maximum contributes 2^0
+
+    // ---- p8 = rne(e * r), four keys to a dword; O^T = V^T P^T
+    i32x4 oacc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+    {
+        oacc[dt] = i32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+    {
+        __builtin_amdgcn_sched_barrier(0);
+        i32x4 preg = {0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+        {
+            if (kb == NKB - 1 && u >= lastTiles)
+            {
+                continue;
+            }
             uint32_t yb[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
-                int const bits = __float_as_int(mul_rounded((float) oacc[dt][j], a.scaleBmm2) + kMagic);
-                yb[j] = (uint32_t) min(max(bits, kMagicBits - 128), kMagicBits + 127);
+                yb[j] = __float_as_uint(fmaf(__int_as_float(acc[kb * 4 + u][j]), r, kMagic));
             }
             uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
             uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
-            pk[dt] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            preg[u] = (int) __builtin_amdgcn_perm(hi, lo, 0x05040100u);
         }
-        rows_transpose(pk);
-        if (qValid)
+        if (DEBUG && a.dbgP8 && qValid)
         {
-            uint8_t* dst = static_cast<uint8_t*>(a.out);
-            int const d0 = g * 16;
-            int64_t off;
-            if (INTERLEAVED)
+            for (int u = 0; u < 4; ++u)
             {
-                off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
+                for (int j = 0; j < 4; ++j)
+                {
+                    int const key = kb * 64 + u * 16 + g * 4 + j;
+                    if (key < sq.nk)
+                    {
+                        a.dbgP8[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
+                            = (int8_t) ((uint32_t) preg[u] >> (8 * j));
+                    }
+                }
             }
-            else
-            {
-                off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
-            }
-            u32x4 const quarter = {pk[0], pk[1], pk[2], pk[3]};
-            *reinterpret_cast<u32x4*>(dst + off) = quarter;
         }
+        int const vrow = kb * 64 + 8 * g + (lq >> 1);
+        uint8_t const* vbase = sV + vrow * kRow + 8 * (lq & 1);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+        {
+            int const sc = swz<1>(vrow, dt) * 16;
+            i32x2 const v0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + sc));
+            i32x2 const v1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + 32 * kRow + sc));
+            i32x4 const vreg = {v0[0], v0[1], v1[0], v1[1]};
+            oacc[dt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vreg, preg, oacc[dt], 0, 0, 0);
+        }
+    }
+
+    // ---- out8 = sat8(rne(acc2 * scale_bmm2)): binary32 product (rounded on its own, not fused
+    //      into the add), rounded to an integer through the magic constant, clamped on the bit
+    //      patterns (monotone for the positive results; anything negative is below the range).
+    //      Lane (g, query) then holds bytes 4g..4g+3 of each 16-byte quarter dt of the query's row; a 4 x 4
+    //      transpose over the four rows of 16 lanes (v_permlane32_swap, v_permlane16_swap) leaves it with the
+    //      whole quarter dt = g, which goes out as one 16-byte store.
+    uint32_t pk[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+    {
+        uint32_t yb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            int const bits = __float_as_int(mul_rounded((float) oacc[dt][j], a.scaleBmm2) + kMagic);
+            yb[j] = (uint32_t) min(max(bits, kMagicBits - 128), kMagicBits + 127);
+        }
+        uint32_t const lo = __builtin_amdgcn_perm(yb[1], yb[0], 0x0c0c0400u);
+        uint32_t const hi = __builtin_amdgcn_perm(yb[3], yb[2], 0x0c0c0400u);
+        pk[dt] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+    }
+    rows_transpose(pk);
+    if (qValid)
+    {
+        uint8_t* dst = static_cast<uint8_t*>(a.out);
+        int const d0 = g * 16;
+        int64_t off;
+        if (INTERLEAVED)
+        {
+            off = (((int64_t) n * 2 + (d0 >> 5)) * a.total + sq.firstTok + q) * 32 + (d0 & 31);
+        }
+        else
+        {
+            off = sq.seqBaseOut + (int64_t) q * a.tokStrideOut + (int64_t) n * kHeadSize + d0;
+        }
+        u32x4 const quarter = {pk[0], pk[1], pk[2], pk[3]};
+        *reinterpret_cast<u32x4*>(dst + off) = quarter;
+    }
+}
+
+// Q^T operand of query tile qt (see tile_i8).
+template <bool INTERLEAVED>
+__device__ __forceinline__ i32x4 load_q_i8(FmhaArgs const& a, SeqInfo const& sq, int const n, int const qt)
+{
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const qq = qt * kQPerWave + (lane & 15);
+    i32x4 v = {0, 0, 0, 0};
+    if (qq < sq.nq)
+    {
+        v = *reinterpret_cast<i32x4 const*>(static_cast<uint8_t const*>(a.qkv)
+            + qkv_chunk_offset<1, INTERLEAVED>(a, sq.seqBaseIn, sq.firstTok, qq, n, 0, lane >> 4));
+    }
+    return v;
+}
+
+// All query tiles of this wavefront for a sequence of exactly NKB key blocks.
+template <int NKB, bool INTERLEAVED, bool DEBUG>
+__device__ __forceinline__ void attend_i8(FmhaArgs const& a, SeqInfo const& sq, int const b, int const n,
+    int const qtBegin, int const qtEnd, uint8_t const* sK, uint8_t const* sV, i32x4 const qFirst)
+{
+    int const wave = threadIdx.x >> 6;
+    constexpr int qtStep = kWavesI8;
+    i32x4 qnext = qFirst; // requested by the caller together with K and V
+    for (int qt = qtBegin + wave; qt < qtEnd; qt += qtStep)
+    {
+        i32x4 const qreg = qnext;
+        qnext = load_q_i8<INTERLEAVED>(a, sq, n, qt + qtStep);
+        tile_i8<NKB, INTERLEAVED, DEBUG>(a, sq, b, n, qt, sK, sV, qreg);
     }
 }
 
@@ -1720,6 +1734,7 @@ int prepare_kt()
 {
     int st = ensure_lds(reinterpret_cast<void const*>(fmha_i8_prefix_kernel<KT, true, false>), "fmha_i8_prefix_interleaved",
         Lds<1>::total(KT));
+
     st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_i8_prefix_kernel<KT, false, false>), "fmha_i8_prefix",
                       Lds<1>::total(KT));
     st = st ? st : ensure_lds(reinterpret_cast<void const*>(fmha_i8_kernel<KT, true, false>), "fmha_i8_interleaved",

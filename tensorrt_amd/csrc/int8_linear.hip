@@ -627,27 +627,6 @@ __device__ __forceinline__ void linear_tile_run(
     }
 }
 
-// 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane i's bytes land at LDS byte
-// address ldsAddr + 16 i, so one instruction of a wavefront fills 1 KB; ldsAddr is wave-uniform and travels in M0.
-// The data never passes through vector registers, and completion is counted by vmcnt like any vector-memory load.
-// Written as inline assembly on purpose: the compiler then neither counts these loads nor orders LDS reads behind
-// them, and the kernel below places its own s_waitcnt where a stage must have landed.
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm" // M0 is named as clobbered on purpose
-__device__ __forceinline__ void load_to_lds16(void const* g, uint32_t ldsAddr)
-{
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(ldsAddr) : "memory", "m0");
-}
-#pragma clang diagnostic pop
-
-// s_waitcnt vmcnt(N) alone (the other counters at their maxima): gfx9 encoding, vmcnt in bits 3:0 and 15:14
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
 // The persistent run of 256 x 256 tiles with the stages brought in by direct-to-LDS loads: a ring of four LDS stage
 // buffers, stage k+3 requested while stage k is multiplied, no staging registers, no LDS-write instructions and
 // nothing for a wavefront to wait for before the barrier except loads issued two steps earlier.  N a multiple of 256
