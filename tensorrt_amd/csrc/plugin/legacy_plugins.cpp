@@ -9,13 +9,19 @@
 //
 // The reference keeps two full implementations of every plugin.  Here a legacy plugin is an adapter
 // around the IPluginV3 object of the matching current version (6/4/5, 5/6/7/8, 4/5/6): every V2 method
-// maps onto one V3 method, and the serialised byte stream is the V3 plugin's serialised field list
-// written out field by field, which deserializePlugin() turns back into a runtime-phase plugin.  The
-// stream layout is this library's own (the reference's is a raw dump of its members, equally private
-// to the library that wrote it).
+// maps onto one V3 method.  serialize() writes the byte layout of the reference's legacy classes (their
+// members in the order and widths of their serialize() functions: bool 1 byte, int32_t / DataType / float 4,
+// size_t 8, weights as raw arrays, no padding; plugin/common/serialize.hpp:43-65, bertCommon.h:219-225), built
+// from the V3 plugin's serialised field list; deserializePlugin() reads that layout back into the field list
+// that creates the runtime-phase V3 plugin.
+//   embLayerNormPluginLegacy.cpp (serialize), embLayerNormVarSeqlenPluginLegacy.cpp:544-562,
+//   skipLayerNormPluginLegacy.cpp:381-402, skipLayerNormInt8InterleavedPluginLegacy.cpp (serialize),
+//   qkvToContextPluginLegacy.cpp:399-422, 909-925, qkvToContextInt8InterleavedPluginLegacy.cpp (serialize),
+//   runner state: mhaRunner.cu:456-507.
 #include "plugin_base.h"
 
 #include <cstring>
+#include <deque>
 #include <memory>
 #include <string>
 #include <vector>
@@ -27,132 +33,435 @@ namespace plugin
 namespace
 {
 
-constexpr uint32_t kStreamMagic = 0x32564C50; // "PLV2"
-
-size_t fieldElementSize(PluginFieldType t)
+enum class Layout
 {
-    switch (t)
-    {
-    case PluginFieldType::kFLOAT16: return 2;
-    case PluginFieldType::kFLOAT32: return 4;
-    case PluginFieldType::kFLOAT64: return 8;
-    case PluginFieldType::kINT8: return 1;
-    case PluginFieldType::kINT16: return 2;
-    case PluginFieldType::kINT32: return 4;
-    case PluginFieldType::kCHAR: return 1;
-    case PluginFieldType::kDIMS: return sizeof(Dims);
-    case PluginFieldType::kBF16: return 2;
-    case PluginFieldType::kINT64: return 8;
-    case PluginFieldType::kFP8: return 1;
-    case PluginFieldType::kINT4: return 1;
-    case PluginFieldType::kFP4: return 1;
-    case PluginFieldType::kUNKNOWN: return 1; // raw bytes (the attention plugins' runner state)
-    default: return 0;
-    }
-}
-
-size_t pad8(size_t n)
-{
-    return (n + 7) & ~size_t(7);
-}
-
-// [magic u32][nbFields u32] then per field [nameLen u32][type i32][length i32][pad u32][name, padded to 8]
-// [data, padded to 8]
-size_t streamSize(PluginFieldCollection const& fc)
-{
-    size_t n = 8;
-    for (int32_t i = 0; i < fc.nbFields; ++i)
-    {
-        PluginField const& f = fc.fields[i];
-        n += 16 + pad8(std::strlen(f.name)) + pad8(fieldElementSize(f.type) * static_cast<size_t>(f.length));
-    }
-    return n;
-}
-
-void writeStream(PluginFieldCollection const& fc, uint8_t* out)
-{
-    auto put32 = [&](uint32_t v) {
-        std::memcpy(out, &v, 4);
-        out += 4;
-    };
-    put32(kStreamMagic);
-    put32(static_cast<uint32_t>(fc.nbFields));
-    for (int32_t i = 0; i < fc.nbFields; ++i)
-    {
-        PluginField const& f = fc.fields[i];
-        size_t const nameLen = std::strlen(f.name);
-        size_t const bytes = fieldElementSize(f.type) * static_cast<size_t>(f.length);
-        put32(static_cast<uint32_t>(nameLen));
-        put32(static_cast<uint32_t>(f.type));
-        put32(static_cast<uint32_t>(f.length));
-        put32(0);
-        std::memset(out, 0, pad8(nameLen));
-        std::memcpy(out, f.name, nameLen);
-        out += pad8(nameLen);
-        std::memset(out, 0, pad8(bytes));
-        if (bytes)
-        {
-            std::memcpy(out, f.data, bytes);
-        }
-        out += pad8(bytes);
-    }
-}
-
-// Parsed stream: owns the names; data pointers refer into the caller's buffer (8-byte aligned offsets).
-struct ParsedStream
-{
-    std::vector<std::string> names;
-    std::vector<PluginField> fields;
-    PluginFieldCollection fc{};
+    kEMB_FIXED,        // CustomEmbLayerNormPluginDynamic 1
+    kEMB_VARSEQLEN,    // 2 (HFace), 3 (MTron)
+    kSKIP,             // CustomSkipLayerNormPluginDynamic 1, 2
+    kSKIP_INTERLEAVED, // 3, 4
+    kQKV,              // CustomQKVToContextPluginDynamic 1
+    kQKV_VARSEQLEN,    // 2
+    kQKV_INTERLEAVED,  // 3
 };
 
-void parseStream(void const* data, size_t length, ParsedStream& ps)
+// What the legacy classes keep as members that the V3 field lists do not carry.
+struct Extras
 {
-    auto const* p = static_cast<uint8_t const*>(data);
-    auto const* end = p + length;
-    auto need = [&](size_t n) {
-        if (static_cast<size_t>(end - p) < n)
+    int64_t S{0};   // EmbLayerNorm 1: the sequence length seen by configurePlugin
+    bool mtron{false};
+};
+
+class ByteWriter
+{
+public:
+    template <typename T>
+    void put(T v)
+    {
+        auto const* p = reinterpret_cast<uint8_t const*>(&v);
+        mBuf.insert(mBuf.end(), p, p + sizeof(T));
+    }
+    void bytes(void const* p, size_t n)
+    {
+        auto const* b = static_cast<uint8_t const*>(p);
+        mBuf.insert(mBuf.end(), b, b + n);
+    }
+    std::vector<uint8_t> const& data() const
+    {
+        return mBuf;
+    }
+
+private:
+    std::vector<uint8_t> mBuf;
+};
+
+class ByteReader
+{
+public:
+    ByteReader(void const* data, size_t length)
+        : mP(static_cast<uint8_t const*>(data))
+        , mEnd(mP + (data ? length : 0))
+    {
+        if (data == nullptr)
         {
             throw std::runtime_error("serialised plugin is truncated");
         }
-    };
-    auto get32 = [&]() {
-        need(4);
-        uint32_t v;
-        std::memcpy(&v, p, 4);
-        p += 4;
+    }
+    template <typename T>
+    T get()
+    {
+        T v;
+        std::memcpy(&v, span(sizeof(T)), sizeof(T));
         return v;
+    }
+    bool flag()
+    {
+        return get<uint8_t>() != 0;
+    }
+    uint8_t const* span(size_t n)
+    {
+        if (static_cast<size_t>(mEnd - mP) < n)
+        {
+            throw std::runtime_error("serialised plugin is truncated");
+        }
+        uint8_t const* p = mP;
+        mP += n;
+        return p;
+    }
+    // element counts come from the stream: refuse what cannot fit before multiplying
+    size_t count(uint64_t n, size_t elemBytes)
+    {
+        if (n > static_cast<uint64_t>(mEnd - mP) / (elemBytes ? elemBytes : 1))
+        {
+            throw std::runtime_error("serialised plugin is truncated");
+        }
+        return static_cast<size_t>(n);
+    }
+
+private:
+    uint8_t const* mP;
+    uint8_t const* mEnd;
+};
+
+// The field list handed to createPlugin(kRUNTIME): owns its values (8-byte aligned copies, because nothing in the
+// reference's byte layout is aligned).
+class FieldStore
+{
+public:
+    void i32(char const* name, int32_t v)
+    {
+        raw(name, &v, 4, PluginFieldType::kINT32, 1);
+    }
+    void f32(char const* name, float v)
+    {
+        raw(name, &v, 4, PluginFieldType::kFLOAT32, 1);
+    }
+    void raw(char const* name, void const* p, size_t bytes, PluginFieldType type, int32_t length)
+    {
+        mBlobs.emplace_back((bytes + 7) / 8 + 1);
+        std::memcpy(mBlobs.back().data(), p, bytes);
+        mFields.emplace_back(name, mBlobs.back().data(), type, length);
+    }
+    PluginFieldCollection collection()
+    {
+        return PluginFieldCollection{static_cast<int32_t>(mFields.size()), mFields.data()};
+    }
+
+private:
+    std::deque<std::vector<uint64_t>> mBlobs;
+    std::vector<PluginField> mFields;
+};
+
+PluginField const* fieldOf(PluginFieldCollection const& fc, char const* name)
+{
+    for (int32_t i = 0; i < fc.nbFields; ++i)
+    {
+        if (fc.fields[i].name && std::strcmp(fc.fields[i].name, name) == 0 && fc.fields[i].data)
+        {
+            return &fc.fields[i];
+        }
+    }
+    return nullptr;
+}
+
+int32_t i32Of(PluginFieldCollection const& fc, char const* name, int32_t fallback)
+{
+    PluginField const* f = fieldOf(fc, name);
+    return f && f->type == PluginFieldType::kINT32 && f->length >= 1 ? *static_cast<int32_t const*>(f->data) : fallback;
+}
+
+float f32Of(PluginFieldCollection const& fc, char const* name, float fallback)
+{
+    PluginField const* f = fieldOf(fc, name);
+    return f && f->type == PluginFieldType::kFLOAT32 && f->length >= 1 ? *static_cast<float const*>(f->data) : fallback;
+}
+
+size_t weightBytes(PluginField const& f)
+{
+    return static_cast<size_t>(f.length) * (f.type == PluginFieldType::kFLOAT16 ? 2 : 4);
+}
+
+PluginField const& required(PluginFieldCollection const& fc, char const* name)
+{
+    PluginField const* f = fieldOf(fc, name);
+    if (!f)
+    {
+        throw std::runtime_error(std::string("the plugin does not serialise its field ") + name);
+    }
+    return *f;
+}
+
+constexpr char const* kEMB_BETA = "bert_embeddings_layernorm_beta";
+constexpr char const* kEMB_GAMMA = "bert_embeddings_layernorm_gamma";
+constexpr char const* kEMB_WORD = "bert_embeddings_word_embeddings";
+constexpr char const* kEMB_TOK = "bert_embeddings_token_type_embeddings";
+constexpr char const* kEMB_POS = "bert_embeddings_position_embeddings";
+
+// ---- V3 field list -> the legacy class's bytes ---------------------------------------------------------------
+std::vector<uint8_t> encode(Layout layout, PluginFieldCollection const& fc, Extras const& ex)
+{
+    ByteWriter w;
+    auto const half = static_cast<int32_t>(DataType::kHALF);
+    auto const flt = static_cast<int32_t>(DataType::kFLOAT);
+    switch (layout)
+    {
+    case Layout::kEMB_FIXED:
+    case Layout::kEMB_VARSEQLEN:
+    {
+        PluginField const& beta = required(fc, kEMB_BETA);
+        PluginField const& gamma = required(fc, kEMB_GAMMA);
+        PluginField const& word = required(fc, kEMB_WORD);
+        PluginField const& pos = required(fc, kEMB_POS);
+        PluginField const& tok = required(fc, kEMB_TOK);
+        int32_t const type = i32Of(fc, "output_fp16", 0) ? half : flt;
+        uint64_t const ld = static_cast<uint64_t>(beta.length);
+        uint64_t const wv = ld ? word.length / ld : 0, pv = ld ? pos.length / ld : 0, tv = ld ? tok.length / ld : 0;
+        w.put<int32_t>(type);                                              // mType
+        if (layout == Layout::kEMB_FIXED)
+        {
+            w.put<int32_t>(i32Of(fc, "mha_type_id", flt));                 // mMhaType
+            w.put<uint64_t>(ld);                                           // mLd
+            w.put<uint64_t>(static_cast<uint64_t>(ex.S));                  // mS
+            w.put<uint64_t>(wv);                                           // mWordVocabSize
+            w.put<uint64_t>(pv);                                           // mPosVocabSize
+            w.put<uint64_t>(tv);                                           // mTokVocabSize
+            w.put<uint8_t>(i32Of(fc, "full_mask", 0) != 0);                // mUseFullMask
+            w.put<int32_t>(getSmVersion());                                // mSM
+        }
+        else
+        {
+            w.put<uint64_t>(ld);
+            w.put<uint64_t>(wv);
+            w.put<uint64_t>(pv);
+            w.put<uint64_t>(tv);
+            w.put<int32_t>(ex.mtron ? type : static_cast<int32_t>(DataType::kINT32)); // mMaskType
+        }
+        w.bytes(beta.data, weightBytes(beta));                             // binary32 [ld]
+        w.bytes(gamma.data, weightBytes(gamma));
+        w.bytes(word.data, weightBytes(word));                             // mType [vocab][ld]
+        w.bytes(pos.data, weightBytes(pos));
+        w.bytes(tok.data, weightBytes(tok));
+        break;
+    }
+    case Layout::kSKIP:
+    {
+        PluginField const& beta = required(fc, "beta");
+        PluginField const& gamma = required(fc, "gamma");
+        PluginField const* bias = fieldOf(fc, "bias");
+        int32_t const type = i32Of(fc, "type_id", flt);
+        w.put<int32_t>(type);                                              // mType
+        w.put<int32_t>(beta.type == PluginFieldType::kFLOAT16 ? half : flt); // mCfgType
+        w.put<uint64_t>(static_cast<uint64_t>(beta.length));               // mLd
+        w.put<uint8_t>(bias != nullptr);                                   // mHasBias
+        w.bytes(beta.data, weightBytes(beta));
+        w.bytes(gamma.data, weightBytes(gamma));
+        if (bias)
+        {
+            w.bytes(bias->data, weightBytes(*bias));
+        }
+        break;
+    }
+    case Layout::kSKIP_INTERLEAVED:
+    {
+        PluginField const& beta = required(fc, "beta");
+        PluginField const& gamma = required(fc, "gamma");
+        w.put<uint64_t>(static_cast<uint64_t>(beta.length));               // mLd
+        w.bytes(beta.data, weightBytes(beta));                             // binary16 [ld]
+        w.bytes(gamma.data, weightBytes(gamma));
+        break;
+    }
+    case Layout::kQKV:
+    case Layout::kQKV_VARSEQLEN:
+    {
+        int32_t const hidden = i32Of(fc, "hidden_size", 0), heads = i32Of(fc, "num_heads", 0);
+        w.put<int32_t>(i32Of(fc, "type_id", flt));                         // mType
+        w.put<int32_t>(heads);                                             // mNumHeads
+        w.put<int32_t>(heads > 0 ? hidden / heads : 0);                    // mHeadSize
+        w.put<uint8_t>(i32Of(fc, "has_mask", 0) != 0);                     // mHasImask
+        w.put<int32_t>(hidden);                                            // mHiddenSize
+        w.put<int32_t>(i32Of(fc, "SM", getSmVersion()));                   // mSM
+        w.put<int32_t>(i32Of(fc, "S", 0));                                 // mS
+        w.put<int32_t>(i32Of(fc, "B", 0));                                 // mB
+        w.put<float>(f32Of(fc, "dq_probs", -1.F));                         // mDqProbs
+        PluginField const* runner = fieldOf(fc, "runnerStateBuffer");
+        if (layout == Layout::kQKV)
+        {
+            bool const has = runner != nullptr && i32Of(fc, "hasUnfusedDispatcher", 0) != 0;
+            w.put<int32_t>(has ? 1 : 0);                                   // hasUnfusedRunner
+            if (has)
+            {
+                w.bytes(runner->data, static_cast<size_t>(runner->length)); // algo1, algo2, S, B, headSize
+            }
+        }
+        else
+        {
+            bool const varSeqlen = i32Of(fc, "var_seqlen", 0) != 0;
+            w.put<uint8_t>(varSeqlen);                                     // mUseVarSeqlen
+            w.put<int32_t>(varSeqlen ? 1 : 2);                             // mHdim
+            w.put<uint8_t>(i32Of(fc, "use_int8_scale_max", 1) != 0);       // mUseInt8ScaleMax
+            if (!runner)
+            {
+                throw std::runtime_error("the attention plugin has no runner yet (configurePlugin first)");
+            }
+            w.bytes(runner->data, static_cast<size_t>(runner->length));    // S, B, headSize (after algo1, algo2 if unfused)
+        }
+        break;
+    }
+    case Layout::kQKV_INTERLEAVED:
+    {
+        int32_t const hidden = i32Of(fc, "hidden_size", 0), heads = i32Of(fc, "num_heads", 0);
+        w.put<int32_t>(heads);                                             // mNumHeads
+        w.put<int32_t>(heads > 0 ? hidden / heads : 0);                    // mHeadSize
+        w.put<int32_t>(hidden);                                            // mHiddenSize
+        w.put<int32_t>(getSmVersion());                                    // mSM
+        w.put<int32_t>(0);                                                 // mS (never set by the reference either)
+        w.put<int32_t>(0);                                                 // mB
+        w.put<float>(f32Of(fc, "dq_probs", -1.F));                         // mDqProbs
+        w.put<uint8_t>(i32Of(fc, "use_int8_scale_max", 1) != 0);           // mUseInt8ScaleMax
+        w.put<uint8_t>(i32Of(fc, "use_explicit_int8", 0) != 0);            // mUseExplicitInt8
+        w.put<float>(f32Of(fc, "input_qkv_scale", 0.F));                   // mQkvScale
+        w.put<float>(f32Of(fc, "output_ctx_scale", 0.F));                  // mCtxScale
+        break;
+    }
+    }
+    return w.data();
+}
+
+// ---- the legacy class's bytes -> the field list of the runtime-phase V3 plugin --------------------------------
+void decode(Layout layout, void const* data, size_t length, FieldStore& fs, Extras& ex)
+{
+    ByteReader r(data, length);
+    auto const half = static_cast<int32_t>(DataType::kHALF);
+    auto weights = [&](char const* name, uint64_t n, bool fp16) {
+        size_t const eb = fp16 ? 2 : 4;
+        size_t const cnt = r.count(n, eb);
+        if (cnt > 0x7fffffffULL)
+        {
+            throw std::runtime_error("serialised plugin holds a weight array beyond 2^31 elements");
+        }
+        fs.raw(name, r.span(cnt * eb), cnt * eb, fp16 ? PluginFieldType::kFLOAT16 : PluginFieldType::kFLOAT32,
+            static_cast<int32_t>(cnt));
     };
-    if (data == nullptr || get32() != kStreamMagic)
+    switch (layout)
     {
-        throw std::runtime_error("not a plugin stream written by this library");
-    }
-    uint32_t const n = get32();
-    if (static_cast<size_t>(n) > length / 16)
+    case Layout::kEMB_FIXED:
+    case Layout::kEMB_VARSEQLEN:
     {
-        throw std::runtime_error("serialised plugin is truncated"); // every field takes at least its 16-byte header
+        int32_t const type = r.get<int32_t>();
+        bool const fp16 = type == half;
+        uint64_t ld, wv, pv, tv;
+        if (layout == Layout::kEMB_FIXED)
+        {
+            fs.i32("mha_type_id", r.get<int32_t>());
+            ld = r.get<uint64_t>();
+            ex.S = static_cast<int64_t>(r.get<uint64_t>());
+            wv = r.get<uint64_t>();
+            pv = r.get<uint64_t>();
+            tv = r.get<uint64_t>();
+            fs.i32("full_mask", r.flag() ? 1 : 0);
+            (void) r.get<int32_t>(); // mSM: the architecture the stream was written on
+        }
+        else
+        {
+            ld = r.get<uint64_t>();
+            wv = r.get<uint64_t>();
+            pv = r.get<uint64_t>();
+            tv = r.get<uint64_t>();
+            (void) r.get<int32_t>(); // mMaskType follows from the version
+        }
+        fs.i32("output_fp16", fp16 ? 1 : 0);
+        size_t const n = r.count(ld, 4);
+        weights(kEMB_BETA, n, false);
+        weights(kEMB_GAMMA, n, false);
+        size_t const eb = fp16 ? 2 : 4;
+        weights(kEMB_WORD, static_cast<uint64_t>(n) * r.count(wv, n * eb ? n * eb : 1), fp16);
+        weights(kEMB_POS, static_cast<uint64_t>(n) * r.count(pv, n * eb ? n * eb : 1), fp16);
+        weights(kEMB_TOK, static_cast<uint64_t>(n) * r.count(tv, n * eb ? n * eb : 1), fp16);
+        break;
     }
-    ps.names.reserve(n);
-    for (uint32_t i = 0; i < n; ++i)
+    case Layout::kSKIP:
     {
-        uint32_t const nameLen = get32();
-        auto const type = static_cast<PluginFieldType>(get32());
-        auto const len = static_cast<int32_t>(get32());
-        get32();
-        need(pad8(nameLen));
-        ps.names.emplace_back(reinterpret_cast<char const*>(p), nameLen);
-        p += pad8(nameLen);
-        size_t const bytes = fieldElementSize(type) * static_cast<size_t>(len < 0 ? 0 : len);
-        need(pad8(bytes));
-        ps.fields.emplace_back(nullptr, bytes ? p : nullptr, type, len);
-        p += pad8(bytes);
+        fs.i32("type_id", r.get<int32_t>());
+        bool const fp16 = r.get<int32_t>() == half;
+        uint64_t const ld = r.get<uint64_t>();
+        bool const hasBias = r.flag();
+        if (ld > 0x7fffffffULL)
+        {
+            throw std::runtime_error("serialised plugin is truncated");
+        }
+        fs.i32("ld", static_cast<int32_t>(ld));
+        weights("beta", ld, fp16);
+        weights("gamma", ld, fp16);
+        if (hasBias)
+        {
+            weights("bias", ld, fp16);
+        }
+        break;
     }
-    for (size_t i = 0; i < ps.fields.size(); ++i)
+    case Layout::kSKIP_INTERLEAVED:
     {
-        ps.fields[i].name = ps.names[i].c_str();
+        uint64_t const ld = r.get<uint64_t>();
+        weights("beta", ld, true);
+        weights("gamma", ld, true);
+        break;
     }
-    ps.fc.nbFields = static_cast<int32_t>(ps.fields.size());
-    ps.fc.fields = ps.fields.data();
+    case Layout::kQKV:
+    case Layout::kQKV_VARSEQLEN:
+    {
+        int32_t const type = r.get<int32_t>();
+        fs.i32("type_id", type);
+        fs.i32("num_heads", r.get<int32_t>());
+        (void) r.get<int32_t>(); // mHeadSize = hidden / heads
+        fs.i32("has_mask", r.flag() ? 1 : 0);
+        fs.i32("hidden_size", r.get<int32_t>());
+        int32_t const sm = r.get<int32_t>();
+        fs.i32("S", r.get<int32_t>());
+        fs.i32("B", r.get<int32_t>());
+        float const dqProbs = r.get<float>();
+        if (dqProbs >= 0.F)
+        {
+            fs.f32("dq_probs", dqProbs);
+        }
+        if (layout == Layout::kQKV)
+        {
+            fs.i32("SM", sm);
+            int32_t const has = r.get<int32_t>();
+            fs.i32("hasUnfusedDispatcher", has != 0 ? 1 : 0);
+            if (has != 0)
+            {
+                fs.raw("runnerStateBuffer", r.span(20), 20, PluginFieldType::kUNKNOWN, 20);
+            }
+        }
+        else
+        {
+            bool const varSeqlen = r.flag();
+            fs.i32("var_seqlen", varSeqlen ? 1 : 0);
+            (void) r.get<int32_t>(); // mHdim follows from var_seqlen
+            fs.i32("use_int8_scale_max", r.flag() ? 1 : 0);
+            size_t const n = varSeqlen ? 12 : 20; // fused runner: S, B, headSize; unfused: two algorithms first
+            fs.raw("runnerStateBuffer", r.span(n), n, PluginFieldType::kUNKNOWN, static_cast<int32_t>(n));
+        }
+        break;
+    }
+    case Layout::kQKV_INTERLEAVED:
+    {
+        fs.i32("num_heads", r.get<int32_t>());
+        (void) r.get<int32_t>();
+        fs.i32("hidden_size", r.get<int32_t>());
+        (void) r.get<int32_t>(); // mSM
+        (void) r.get<int32_t>(); // mS
+        (void) r.get<int32_t>(); // mB
+        float const dqProbs = r.get<float>();
+        if (dqProbs >= 0.F)
+        {
+            fs.f32("dq_probs", dqProbs);
+        }
+        fs.i32("use_int8_scale_max", r.flag() ? 1 : 0);
+        fs.i32("use_explicit_int8", r.flag() ? 1 : 0);
+        fs.f32("input_qkv_scale", r.get<float>());
+        fs.f32("output_ctx_scale", r.get<float>());
+        break;
+    }
+    }
 }
 
 struct V3Deleter
@@ -184,11 +493,14 @@ std::vector<DynamicPluginTensorDesc> widen(PluginTensorDesc const* d, int32_t n)
 class LegacyAdapter final : public IPluginV2DynamicExt
 {
 public:
-    LegacyAdapter(V3Ptr plugin, char const* legacyVersion, std::string ns, int32_t nbInputs)
+    LegacyAdapter(V3Ptr plugin, char const* legacyVersion, std::string ns, int32_t nbInputs, Layout layout,
+        Extras const& extras)
         : mPlugin(std::move(plugin))
         , mVersion(legacyVersion)
         , mNamespace(std::move(ns))
         , mNbInputs(nbInputs)
+        , mLayout(layout)
+        , mExtras(extras)
     {
         mCore = cap<IPluginV3OneCore>(mPlugin.get(), PluginCapabilityType::kCORE);
         mBuild = cap<IPluginV3OneBuild>(mPlugin.get(), PluginCapabilityType::kBUILD);
@@ -215,15 +527,14 @@ public:
     void terminate() noexcept override {}
     size_t getSerializationSize() const noexcept override
     {
-        PluginFieldCollection const* fc = mRuntime->getFieldsToSerialize();
-        return fc ? streamSize(*fc) : 0;
+        return encoded().size();
     }
     void serialize(void* buffer) const noexcept override
     {
-        PluginFieldCollection const* fc = mRuntime->getFieldsToSerialize();
-        if (fc && buffer)
+        std::vector<uint8_t> const bytes = encoded();
+        if (buffer && !bytes.empty())
         {
-            writeStream(*fc, static_cast<uint8_t*>(buffer));
+            std::memcpy(buffer, bytes.data(), bytes.size());
         }
     }
     void destroy() noexcept override
@@ -267,7 +578,7 @@ public:
             {
                 return nullptr;
             }
-            return new LegacyAdapter(std::move(copy), mVersion, mNamespace, mNbInputs);
+            return new LegacyAdapter(std::move(copy), mVersion, mNamespace, mNbInputs, mLayout, mExtras);
         }
         catch (...)
         {
@@ -306,6 +617,10 @@ public:
         int32_t nbOutputs) noexcept override
     {
         mNbInputs = nbInputs;
+        if (mLayout == Layout::kEMB_FIXED && in && nbInputs > 0 && in[0].desc.dims.nbDims > 0)
+        {
+            mExtras.S = in[0].desc.dims.d[0]; // [S, B]: what the legacy class keeps as mS
+        }
         mBuild->configurePlugin(in, nbInputs, out, nbOutputs);
     }
     size_t getWorkspaceSize(PluginTensorDesc const* inputs, int32_t nbInputs, PluginTensorDesc const* outputs,
@@ -336,6 +651,29 @@ public:
     }
 
 private:
+    std::vector<uint8_t> encoded() const noexcept
+    {
+        try
+        {
+            PluginFieldCollection const* fc = mRuntime->getFieldsToSerialize();
+            if (fc)
+            {
+                return encode(mLayout, *fc, mExtras);
+            }
+        }
+        catch (std::exception const& e)
+        {
+            if (ILogger* l = getLogger())
+            {
+                l->log(ILogger::Severity::kERROR, e.what());
+            }
+        }
+        catch (...)
+        {
+        }
+        return {};
+    }
+
     V3Ptr mPlugin;
     IPluginV3OneCore* mCore{};
     IPluginV3OneBuild* mBuild{};
@@ -343,7 +681,24 @@ private:
     char const* mVersion;
     std::string mNamespace;
     int32_t mNbInputs;
+    Layout mLayout;
+    Extras mExtras;
 };
+
+Layout layoutOf(char const* pluginName, char const* legacyVersion)
+{
+    std::string const name = pluginName;
+    int const v = std::atoi(legacyVersion);
+    if (name == "CustomSkipLayerNormPluginDynamic")
+    {
+        return v <= 2 ? Layout::kSKIP : Layout::kSKIP_INTERLEAVED;
+    }
+    if (name == "CustomEmbLayerNormPluginDynamic")
+    {
+        return v == 1 ? Layout::kEMB_FIXED : Layout::kEMB_VARSEQLEN;
+    }
+    return v == 1 ? Layout::kQKV : (v == 2 ? Layout::kQKV_VARSEQLEN : Layout::kQKV_INTERLEAVED);
+}
 
 // How many inputs each operator takes, from its serialised configuration (needed because the V2
 // enqueue() does not say): SkipLayerNorm 2; EmbLayerNorm fixed 3, var-seqlen 4; QKV-to-context 1 + has_mask
@@ -408,15 +763,17 @@ public:
     }
     IPluginV2* createPlugin(AsciiChar const* name, PluginFieldCollection const* fc) noexcept override
     {
-        return make(name, fc, TensorRTPhase::kBUILD);
+        return make(name, fc, TensorRTPhase::kBUILD, Extras{});
     }
     IPluginV2* deserializePlugin(AsciiChar const* name, void const* serialData, size_t serialLength) noexcept override
     {
         try
         {
-            ParsedStream ps;
-            parseStream(serialData, serialLength, ps);
-            return make(name, &ps.fc, TensorRTPhase::kRUNTIME);
+            FieldStore fs;
+            Extras ex;
+            decode(layoutOf(mName, mVersion), serialData, serialLength, fs, ex);
+            PluginFieldCollection const fc = fs.collection();
+            return make(name, &fc, TensorRTPhase::kRUNTIME, ex);
         }
         catch (std::exception const& e)
         {
@@ -448,7 +805,7 @@ private:
     {
         return static_cast<IPluginCreatorV3One*>(getPluginRegistry()->getCreator(mName, mCurrent, ""));
     }
-    IPluginV2* make(AsciiChar const* name, PluginFieldCollection const* fc, TensorRTPhase phase) noexcept
+    IPluginV2* make(AsciiChar const* name, PluginFieldCollection const* fc, TensorRTPhase phase, Extras ex) noexcept
     {
         try
         {
@@ -464,7 +821,8 @@ private:
                 return nullptr; // the V3 creator has logged why
             }
             int32_t const nbIn = inputsOf(mName, mVersion, p.get());
-            return new LegacyAdapter(std::move(p), mVersion, mNamespace, nbIn);
+            ex.mtron = std::string(mName) == "CustomEmbLayerNormPluginDynamic" && std::atoi(mVersion) == 3;
+            return new LegacyAdapter(std::move(p), mVersion, mNamespace, nbIn, layoutOf(mName, mVersion), ex);
         }
         catch (std::exception const& e)
         {

@@ -523,6 +523,108 @@ def test_legacy_versions_wrap_the_current_plugins(reg, name, legacy, current):
     last_log()
 
 
+def test_legacy_streams_have_the_reference_byte_layout(reg):
+    """serialize() writes the members of the reference's legacy classes in the order and widths of their own
+    serialize() functions (bool 1 byte, int32_t / DataType / float 4, size_t 8, weights raw, no padding).  The
+    expected bytes are put together by hand here, one plugin of each family and layout."""
+    import struct
+    r = np.random.default_rng(11)
+    HALF, FLOAT, INT32 = 1, 0, 3
+    SM = 80
+
+    # SkipLayerNorm 1 (skipLayerNormPluginLegacy.cpp:381-402): mType, mCfgType, mLd, mHasBias, beta, gamma, bias
+    ld = 64
+    beta, gamma, bias = (r.standard_normal(ld).astype(np.float32) for _ in range(3))
+    lc = reg.get_legacy_creator(SKIPLN, "1")
+    p = lc.create_plugin("l", [PluginField("beta", beta, F32), PluginField("gamma", gamma, F32),
+                               PluginField("bias", bias, F32), i32("type_id", HALF), i32("ld", ld)])
+    want = struct.pack("<iiQB", HALF, HALF, ld, 1) + b"".join(a.astype(np.float16).tobytes() for a in (beta, gamma, bias))
+    assert p.serialize() == want
+    p = lc.create_plugin("l", [PluginField("beta", beta, F32), PluginField("gamma", gamma, F32), i32("type_id", FLOAT),
+                               i32("ld", ld)])
+    assert p.serialize() == struct.pack("<iiQB", FLOAT, FLOAT, ld, 0) + beta.tobytes() + gamma.tobytes()
+    q = lc.deserialize_plugin("l", want)
+    assert q is not None and q.serialize() == want
+
+    # SkipLayerNorm 3 (skipLayerNormInt8InterleavedPluginLegacy.cpp): mLd, beta, gamma in binary16
+    p = reg.get_legacy_creator(SKIPLN, "3").create_plugin("l", [PluginField("beta", beta, F32), PluginField("gamma", gamma, F32)])
+    assert p.serialize() == struct.pack("<Q", ld) + beta.astype(np.float16).tobytes() + gamma.astype(np.float16).tobytes()
+
+    # EmbLayerNorm 1 (embLayerNormPluginLegacy.cpp): mType, mMhaType, mLd, mS, three vocabulary sizes, mUseFullMask,
+    # mSM, beta, gamma (binary32), word, position, token-type tables (mType)
+    E, V, P, T = 32, 10, 16, 2
+    eb, eg = r.standard_normal(E).astype(np.float32), r.standard_normal(E).astype(np.float32)
+    word, pos, tok = (r.standard_normal((n, E)).astype(np.float32) for n in (V, P, T))
+    emb = [PluginField("bert_embeddings_layernorm_beta", eb, F32), PluginField("bert_embeddings_layernorm_gamma", eg, F32),
+           PluginField("bert_embeddings_word_embeddings", word, F32),
+           PluginField("bert_embeddings_token_type_embeddings", tok, F32),
+           PluginField("bert_embeddings_position_embeddings", pos, F32), i32("output_fp16", 1)]
+    lc = reg.get_legacy_creator(EMBLN, "1")
+    p = lc.create_plugin("l", emb + [i32("full_mask", 1), i32("mha_type_id", HALF)])
+    tables = b"".join(a.astype(np.float16).tobytes() for a in (word, pos, tok))
+    head = lambda S: struct.pack("<iiQQQQQBi", HALF, HALF, E, S, V, P, T, 1, SM)
+    assert p.serialize() == head(0) + eb.tobytes() + eg.tobytes() + tables
+    ids = TensorDesc([128, 4], DataType.INT32)
+    p.configure_plugin([ids, ids, ids], [TensorDesc([128, 4, E, 1, 1], DataType.HALF), TensorDesc([4, 512], DataType.INT32)])
+    blob = p.serialize()
+    assert blob == head(128) + eb.tobytes() + eg.tobytes() + tables      # configurePlugin sets mS
+    q = lc.deserialize_plugin("l", blob)
+    assert q is not None and q.serialize() == blob and q.clone().serialize() == blob
+
+    # EmbLayerNorm 2 / 3 (embLayerNormVarSeqlenPluginLegacy.cpp:544-562): mType, mLd, vocabulary sizes, mMaskType
+    for version, mask_type in (("2", INT32), ("3", FLOAT)):
+        fields = emb[:-1] + [i32("output_fp16", 0)]
+        p = reg.get_legacy_creator(EMBLN, version).create_plugin("l", fields)
+        want = struct.pack("<iQQQQi", FLOAT, E, V, P, T, mask_type) + eb.tobytes() + eg.tobytes() + word.tobytes() \
+            + pos.tobytes() + tok.tobytes()
+        assert p.serialize() == want
+
+    # QKV-to-context 1 (qkvToContextPluginLegacy.cpp:399-422): mType, mNumHeads, mHeadSize, mHasImask, mHiddenSize, mSM,
+    # mS, mB, mDqProbs, hasUnfusedRunner, then the unfused runner: two GEMM algorithms, S, B, head size
+    lc = reg.get_legacy_creator(QKV, "1")
+    p = lc.create_plugin("l", [i32("type_id", HALF), i32("hidden_size", 768), i32("num_heads", 12), i32("has_mask", 1)])
+    assert p.serialize() == struct.pack("<iiiBiiiifi", HALF, 12, 64, 1, 768, SM, 0, 0, -1.0, 0)
+    p.configure_plugin([TensorDesc([128, 2, 3 * 768, 1, 1], DataType.HALF), TensorDesc([2, 512], DataType.INT32)],
+                       [TensorDesc([128, 2, 768, 1, 1], DataType.HALF)])
+    # S = 128 has a fused kernel: only that runner is set up, and no runner state is written
+    assert p.serialize() == struct.pack("<iiiBiiiifi", HALF, 12, 64, 1, 768, SM, 128, 2, -1.0, 0)
+    p.configure_plugin([TensorDesc([200, 2, 3 * 768, 1, 1], DataType.HALF), TensorDesc([2, 1], DataType.INT32)],
+                       [TensorDesc([200, 2, 768, 1, 1], DataType.HALF)])
+    blob = p.serialize()
+    assert blob == struct.pack("<iiiBiiiifi", HALF, 12, 64, 1, 768, SM, 200, 2, -1.0, 1) \
+        + struct.pack("<iiiii", 99, 99, 200, 2, 64)          # CUBLAS_GEMM_DEFAULT_TENSOR_OP = 99 twice
+    q = lc.deserialize_plugin("l", blob)
+    assert q is not None and q.serialize() == blob
+
+    # QKV-to-context 2 (:909-925): ..., mDqProbs, mUseVarSeqlen, mHdim, mUseInt8ScaleMax, then the fused runner: S, B,
+    # head size
+    lc = reg.get_legacy_creator(QKV, "2")
+    p = lc.create_plugin("l", [i32("type_id", 2), i32("hidden_size", 1024), i32("num_heads", 16), i32("has_mask", 1),
+                               i32("var_seqlen", 1), f32("dq_probs", 0.5)])
+    p.configure_plugin([TensorDesc([300, 3 * 1024, 1, 1], DataType.INT8, TensorFormat.CHW32, 0.1), TensorDesc([1], DataType.INT32),
+                        TensorDesc([5], DataType.INT32), TensorDesc([128], DataType.INT32)],
+                       [TensorDesc([300, 1024, 1, 1], DataType.INT8, TensorFormat.CHW32, 0.1)])
+    blob = p.serialize()
+    # variable sequence length: mS and mB stay unset, the runner holds the placeholder geometry (256, 1) that
+    # configurePlugin gives it (qkvToContextPluginLegacy.cpp, QKVToContextVarSeqlenPluginLegacy::configurePlugin)
+    assert blob == struct.pack("<iiiBiiiifBiB", 2, 16, 64, 1, 1024, SM, 0, 0, 0.5, 1, 1, 1) + struct.pack("<iii", 256, 1, 64)
+    q = lc.deserialize_plugin("l", blob)
+    assert q is not None and q.serialize() == blob
+
+    # QKV-to-context 3 (qkvToContextInt8InterleavedPluginLegacy.cpp): heads, head size, hidden, SM, S, B, dq_probs,
+    # use_int8_scale_max, use_explicit_int8, the two explicit scales
+    lc = reg.get_legacy_creator(QKV, "3")
+    p = lc.create_plugin("l", [i32("hidden_size", 1024), i32("num_heads", 16), f32("dq_probs", 0.25),
+                               i32("use_explicit_int8", 1), f32("input_qkv_scale", 0.5), f32("output_ctx_scale", 0.125)])
+    blob = p.serialize()
+    assert blob == struct.pack("<iiiiiifBBff", 16, 64, 1024, SM, 0, 0, 0.25, 1, 1, 0.5, 0.125)
+    q = lc.deserialize_plugin("l", blob)
+    assert q is not None and q.serialize() == blob
+    for cut in (1, 8, len(blob) - 1):
+        assert lc.deserialize_plugin("l", blob[:cut]) is None
+        assert "truncated" in last_log()
+
+
 def test_legacy_skipln_shapes_types_formats(reg):
     lc = reg.get_legacy_creator(SKIPLN, "1")
     p = lc.create_plugin("sln", legacy_fields(SKIPLN, "1"))
