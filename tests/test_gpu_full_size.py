@@ -10,8 +10,8 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (assert_fp_close, assert_int8_close, attention_f64, dev, dev_empty, f32_bits, half2_bits, host, ptr,
-                     quantize_amax, rng, stream, sync)
+from helpers import (assert_fp_close, assert_int8_close, attention_f64, dev, dev_empty, f32_bits, half2_bits, host,
+                     int8_attention_parity, ptr, quantize_amax, rng, stream, sync)
 
 pytestmark = pytest.mark.gpu
 D = 64
@@ -117,15 +117,11 @@ def test_int8_attention_at_benchmark_size(api):
     full = run(qkv, cu)
     # every row was written: a row of the fill pattern would have all 1024 values equal to 0x55
     assert not (full == 0x55).all(axis=1).any()
-    off = total = 0
+    # sampled sequences, run alone: the same bytes as in the batch, first accumulators and second product exact,
+    # probabilities within one step (<= 1e-5 of them off), rows with agreeing probabilities bit-exact
     for b in sample_of(lens, r):
         lo, hi = cu[b], cu[b + 1]
-        ref = oracle.mha_fused_i8_packed(qkv[lo:hi], cu_of(lens[b:b + 1]), N, D, s1, ss, s2)
-        ref = np.asarray(ref[0] if isinstance(ref, tuple) else ref).reshape(hi - lo, N * D)
-        assert_int8_close(full[lo:hi], ref, what=f"sequence {b} vs oracle")
-        off += int((full[lo:hi] != ref).sum())
-        total += ref.size
-    assert off <= 1e-3 * total, f"{off} of {total} outputs differ from the oracle"
+        int8_attention_parity(qkv[lo:hi], cu_of(lens[b:b + 1]), N, s1, ss, s2, interleaved=True, S=S, expect=full[lo:hi])
     order = r.permutation(B)
     moved = run(gather_sequences(qkv, cu, order), cu_of(lens[order]))
     assert np.array_equal(moved, gather_sequences(full, cu, order))
