@@ -170,9 +170,14 @@ int scaled_softmax(hipStream_t stream, int32_t ld, int32_t B, int32_t N, float w
 }
 
 // ------------------------------------------------------------------------------------------
-// Strided batched GEMM on the vector ALU, 64x64 output tile per workgroup, binary32
-// accumulation: C[m,n] = sum_k A(m,k) * B(k,n), operands addressed by element strides so the
-// same kernel serves Q K^T (B = K read along its rows) and P V.
+// Strided batched GEMM on the matrix cores, binary32 accumulation: C[m,n] = sum_k A(m,k) * B(k,n), operands
+// addressed by element strides so the same kernel serves Q K^T (B = K read along its rows) and P V.
+// A workgroup of four wavefronts owns a 64 x 64 tile of C, a wavefront a 32 x 32 quarter of it in one accumulator
+// tile of v_mfma_f32_32x32x16_f16 (binary16 operands) or v_mfma_f32_32x32x2_f32 (binary32 operands: full IEEE
+// multiplies).  k advances in chunks of 32 through LDS, both operands stored [row][k] there, so that a fragment
+// is one 16-byte read (binary16) or one 4-byte read per instruction (binary32); rows and k beyond the matrix are
+// zero in LDS, so any M, N, K is served.  Global reads take 16 bytes per lane along whichever dimension is
+// contiguous when addresses and strides allow, single elements otherwise.
 // Batch index z = b*heads + h; operand base = b*batchStride + h*headStride.
 // ------------------------------------------------------------------------------------------
 struct GemmOperand
@@ -180,85 +185,166 @@ struct GemmOperand
     int64_t batchStride, headStride, rowStride, colStride;
 };
 
+constexpr int kGemmTile = 64; // rows and columns of C per workgroup
+constexpr int kGemmK = 32;    // k per LDS stage
+
+template <typename T>
+struct GemmLds
+{
+    // row pitch in elements: 16-byte aligned rows for the binary16 fragment reads, an odd number of dwords for the
+    // binary32 ones (consecutive rows then fall in consecutive banks)
+    static constexpr int kPitch = sizeof(T) == 2 ? kGemmK + 8 : kGemmK + 1;
+};
+
+// One operand's 64 x 32 stage into LDS as [row][k].  rowStride / kStride are the element strides of the operand's
+// row index (m or n) and of k in global memory; rows < rowsLeft and k < kLeft exist.
+template <typename T>
+__device__ inline void stage_operand(T const* __restrict__ g, int64_t const rowStride, int64_t const kStride,
+    int const rowsLeft, int const kLeft, bool const vec, T* __restrict__ lds)
+{
+    constexpr int P = GemmLds<T>::kPitch;
+    constexpr int V = 16 / sizeof(T); // elements per 16-byte access
+    if (vec && kStride == 1)
+    {
+        // 16 bytes along k: (64 rows) x (32 / V chunks)
+        for (int c = threadIdx.x; c < kGemmTile * (kGemmK / V); c += kBlock)
+        {
+            int const row = c / (kGemmK / V), k0 = (c % (kGemmK / V)) * V;
+            T tmp[V];
+            if (row < rowsLeft && k0 + V <= kLeft)
+            {
+                *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<u32x4 const*>(g + row * rowStride + k0);
+            }
+            else
+            {
+#pragma unroll
+                for (int i = 0; i < V; ++i)
+                {
+                    tmp[i] = (row < rowsLeft && k0 + i < kLeft) ? g[row * rowStride + k0 + i] : (T) 0.f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < V; ++i)
+            {
+                lds[row * P + k0 + i] = tmp[i];
+            }
+        }
+    }
+    else if (vec && rowStride == 1)
+    {
+        // 16 bytes along the row index (V rows of one k): transposed on the way into LDS
+        for (int c = threadIdx.x; c < kGemmK * (kGemmTile / V); c += kBlock)
+        {
+            int const k = c / (kGemmTile / V), r0 = (c % (kGemmTile / V)) * V;
+            T tmp[V];
+            if (k < kLeft && r0 + V <= rowsLeft)
+            {
+                *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<u32x4 const*>(g + k * kStride + r0);
+            }
+            else
+            {
+#pragma unroll
+                for (int i = 0; i < V; ++i)
+                {
+                    tmp[i] = (k < kLeft && r0 + i < rowsLeft) ? g[k * kStride + r0 + i] : (T) 0.f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < V; ++i)
+            {
+                lds[(r0 + i) * P + k] = tmp[i];
+            }
+        }
+    }
+    else
+    {
+        bool const kFastest = kStride <= rowStride;
+        for (int c = threadIdx.x; c < kGemmTile * kGemmK; c += kBlock)
+        {
+            int const row = kFastest ? c / kGemmK : c % kGemmTile;
+            int const k = kFastest ? c % kGemmK : c / kGemmTile;
+            lds[row * P + k] = (row < rowsLeft && k < kLeft) ? g[row * rowStride + k * kStride] : (T) 0.f;
+        }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void batched_gemm_kernel(int const M, int const N, int const K, int const heads,
     T const* __restrict__ A, GemmOperand const oa, T const* __restrict__ B, GemmOperand const ob, T* __restrict__ Cm,
-    GemmOperand const oc)
+    GemmOperand const oc, int const vecA, int const vecB)
 {
-    constexpr int TM = 64, TN = 64, TK = 16;
-    __shared__ float sA[TK][TM + 1];
-    __shared__ float sB[TK][TN + 1];
+    constexpr int P = GemmLds<T>::kPitch;
+    __shared__ __attribute__((aligned(16))) T sA[kGemmTile * P];
+    __shared__ __attribute__((aligned(16))) T sB[kGemmTile * P];
     int const z = blockIdx.z;
     int const b = z / heads, h = z % heads;
     T const* a = A + b * oa.batchStride + h * oa.headStride;
     T const* bb = B + b * ob.batchStride + h * ob.headStride;
     T* c = Cm + b * oc.batchStride + h * oc.headStride;
-    int const m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
-    int const tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    float acc[4][4] = {};
-    for (int k0 = 0; k0 < K; k0 += TK)
+    int const m0 = blockIdx.y * kGemmTile, n0 = blockIdx.x * kGemmTile;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const wave = threadIdx.x >> 6;
+    int const wm = (wave >> 1) * 32, wn = (wave & 1) * 32; // this wavefront's quarter of the tile
+    int const r = lane & 31, kh = lane >> 5;               // fragment row / column and k half
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
     {
-        for (int i = threadIdx.x; i < TM * TK; i += kBlock)
-        {
-            // A tile: consecutive threads walk k (contiguous for Q and P)
-            int const kk = i % TK, mm = i / TK;
-            int const m = m0 + mm, k = k0 + kk;
-            sA[kk][mm] = (m < M && k < K) ? (float) a[m * oa.rowStride + k * oa.colStride] : 0.f;
-        }
-        for (int i = threadIdx.x; i < TN * TK; i += kBlock)
-        {
-            // B(k,n): choose the walk so that the contiguous dimension varies fastest
-            int kk, nn;
-            if (ob.colStride == 1)
-            {
-                nn = i % TN;
-                kk = i / TN;
-            }
-            else
-            {
-                kk = i % TK;
-                nn = i / TK;
-            }
-            int const n = n0 + nn, k = k0 + kk;
-            sB[kk][nn] = (n < N && k < K) ? (float) bb[k * ob.rowStride + n * ob.colStride] : 0.f;
-        }
+        acc[i] = 0.f;
+    }
+    for (int k0 = 0; k0 < K; k0 += kGemmK)
+    {
+        // A(m,k): row index m, B(k,n): row index n (stored [n][k])
+        stage_operand<T>(a + m0 * oa.rowStride + k0 * oa.colStride, oa.rowStride, oa.colStride, M - m0, K - k0,
+            vecA != 0, sA);
+        stage_operand<T>(bb + k0 * ob.rowStride + n0 * ob.colStride, ob.colStride, ob.rowStride, N - n0, K - k0,
+            vecB != 0, sB);
         __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < TK; ++kk)
+        if constexpr (sizeof(T) == 2)
         {
-            float av[4], bv[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int ks = 0; ks < kGemmK; ks += 16)
             {
-                av[i] = sA[kk][ty * 4 + i];
-                bv[i] = sB[kk][tx * 4 + i];
+                f16x8 const fa = *reinterpret_cast<f16x8 const*>(&sA[(wm + r) * P + ks + kh * 8]);
+                f16x8 const fb = *reinterpret_cast<f16x8 const*>(&sB[(wn + r) * P + ks + kh * 8]);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, acc, 0, 0, 0);
             }
+        }
+        else
+        {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int ks = 0; ks < kGemmK; ks += 2)
             {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
-                }
+                float const fa = sA[(wm + r) * P + ks + kh];
+                float const fb = sB[(wn + r) * P + ks + kh];
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc, 0, 0, 0);
             }
         }
         __syncthreads();
     }
+    // accumulator i of lane (r, kh): row 8 (i / 4) + 4 kh + i % 4, column r of the wavefront's quarter
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 16; ++i)
     {
-        int const m = m0 + ty * 4 + i;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
+        int const m = m0 + wm + 8 * (i >> 2) + 4 * kh + (i & 3);
+        int const n = n0 + wn + r;
+        if (m < M && n < N)
         {
-            int const n = n0 + tx * 4 + j;
-            if (m < M && n < N)
-            {
-                c[m * oc.rowStride + n * oc.colStride] = (T) acc[i][j];
-            }
+            c[m * oc.rowStride + n * oc.colStride] = (T) acc[i];
         }
     }
+}
+
+// 16-byte accesses along the contiguous dimension are possible when the base, both strides that get multiplied and
+// the batch / head strides keep every address 16-byte aligned.
+template <typename T>
+int can_vectorise(T const* base, GemmOperand const& o)
+{
+    constexpr int64_t V = 16 / sizeof(T);
+    bool const contiguous = o.colStride == 1 || o.rowStride == 1;
+    int64_t const other = o.colStride == 1 ? o.rowStride : o.colStride;
+    return contiguous && (reinterpret_cast<uintptr_t>(base) & 15u) == 0 && other % V == 0 && o.batchStride % V == 0
+        && o.headStride % V == 0;
 }
 
 template <typename T>
@@ -283,7 +369,8 @@ int unfused_mha(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, 
     GemmOperand const ov{N * strideQKV, strideQKV, ldQKV, 1};   // B(k=key, n=dim) = V[key][dim]
     GemmOperand const oo{(int64_t) N * d, d, ldOut, 1};
     dim3 const g1(ceil_div(S, 64), ceil_div(S, 64), (unsigned) numMats);
-    hipLaunchKernelGGL((batched_gemm_kernel<T>), g1, dim3(kBlock), 0, stream, S, S, d, N, q, oq, k, okT, qk, os);
+    hipLaunchKernelGGL((batched_gemm_kernel<T>), g1, dim3(kBlock), 0, stream, S, S, d, N, q, oq, k, okT, qk, os,
+        can_vectorise(q, oq), can_vectorise(k, okT));
     int st = check_launch("batched_gemm_kernel(QK^T)");
     if (st != 0)
     {
@@ -296,7 +383,8 @@ int unfused_mha(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, 
         return st;
     }
     dim3 const g2(ceil_div(d, 64), ceil_div(S, 64), (unsigned) numMats);
-    hipLaunchKernelGGL((batched_gemm_kernel<T>), g2, dim3(kBlock), 0, stream, S, d, S, N, pp, os, v, ov, output, oo);
+    hipLaunchKernelGGL((batched_gemm_kernel<T>), g2, dim3(kBlock), 0, stream, S, d, S, N, pp, os, v, ov, output, oo,
+        can_vectorise(pp, os), can_vectorise(v, ov));
     return check_launch("batched_gemm_kernel(PV)");
 }
 
