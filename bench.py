@@ -33,14 +33,17 @@ sys.path.insert(0, ROOT)
 METRIC = "BERT-large INT8 S=384 seq/s on 1 GPU; % HBM peak (LN) & % INT8 MFMA peak (MHA)"
 PEAK_INT8_OPS = 5.0e15   # dense INT8 MFMA, op/s
 PEAK_HBM = 8.0e12        # B/s
-# HBM bytes per launch on the default workload, from the FETCH_SIZE / WRITE_SIZE counter runs kept in
-# profiles/ (scaled by what the same counters read for a 256 MiB copy); null for any other workload.
-MHA_TRAFFIC_BYTES = 75_200_000
-LN_TRAFFIC_BYTES = 59_700_000
-# the same for the encoder workload's defaults (B=128, lengths uniform[128,384], seed 1: 33289 tokens)
-ENC_FFN1_TRAFFIC_BYTES = 240_000_000
-ENC_MHA_TRAFFIC_BYTES = 137_700_000
-ENC_LN_TRAFFIC_BYTES = 108_800_000
+
+
+def measured_traffic(workload: str, kernel: str):
+    """HBM-side bytes per launch of `kernel` on the default `workload`, as the FETCH_SIZE / WRITE_SIZE counter runs
+    found them (profiles/traffic.json, written by `python -m tensorrt_amd.profile_summary --update` from those runs
+    and scaled by what the same counters read for a 256 MiB copy); None when no such run is on file."""
+    try:
+        doc = json.load(open(os.path.join(ROOT, "profiles", "traffic.json")))
+        return int(doc[workload]["kernels"][kernel]["traffic_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def f32_bits(x) -> int:
@@ -230,7 +233,7 @@ def run_encoder(args, api, torch):
             "peak": PEAK_INT8_OPS / 1e12,
             "unit": "TOP/s",
             "frac": table[dom]["frac_of_int8_mfma_peak"],
-            "traffic": ENC_FFN1_TRAFFIC_BYTES if default_workload else None,
+            "traffic": measured_traffic("encoder", "ffn1_gemm_gelu") if default_workload else None,
             "avg_launch_us": table[dom]["avg_launch_us"],
             "algorithmic_ops_per_launch": ops[dom][1],
         },
@@ -241,7 +244,7 @@ def run_encoder(args, api, torch):
             "peak": PEAK_INT8_OPS / 1e12,
             "unit": "TOP/s",
             "frac": table["attention"]["frac_of_int8_mfma_peak"],
-            "traffic": ENC_MHA_TRAFFIC_BYTES if default_workload else None,
+            "traffic": measured_traffic("encoder", "attention") if default_workload else None,
             "avg_launch_us": table["attention"]["avg_launch_us"],
             "algorithmic_ops_per_launch": ops["attention"][1],
             # its arithmetic intensity (ops per byte of q, k, v and context) is below the machine's ridge of
@@ -256,7 +259,7 @@ def run_encoder(args, api, torch):
             "peak": PEAK_HBM / 1e9,
             "unit": "GB/s",
             "frac": table["skipln"]["frac_of_hbm_peak"],
-            "traffic": ENC_LN_TRAFFIC_BYTES if default_workload else None,
+            "traffic": measured_traffic("encoder", "skipln") if default_workload else None,
             "avg_launch_us": table["skipln"]["avg_launch_us"],
             "algorithmic_bytes_per_launch": ln_bytes,
         },
@@ -264,8 +267,21 @@ def run_encoder(args, api, torch):
         "sum_of_kernel_times_ms": round(per_layer * cfg.layers * 1e3, 3),
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_encoder(enc, cu, ms_budget_s=20.0)
-        out["cpu_baseline_fp32_library"] = cpu_baseline_torch(enc, cu, lens, torch)
+        out["cpu_baseline"] = cpu_baseline_encoder(enc, cu, ms_budget_s=6.0)
+        out["cpu_baseline_fp32_library"] = cpu_baseline_torch(enc, cu, lens, torch, budget_s=3.0)
+    if not args.no_configs:
+        # the other configurations' kernels at their stated sizes, and this GPU's instruction rates
+        from tensorrt_amd import kernel_bench
+        del enc
+        torch.cuda.empty_cache()
+        out["microbench"] = kernel_bench.microbench(torch)
+        rows = kernel_bench.config_rows(api, torch, steps=100, seed=args.seed, cpu=not args.no_cpu_baseline,
+                                        launch_floor_us=out["microbench"]["empty_launch_us"]["256x256"])
+        out["configs"] = rows
+        cold = [r for r in rows if r["config"] == "C5" and "SkipLN" in r["kernel"]]
+        if cold:
+            out["roofline_skipln"]["cold_cache"] = {"achieved": cold[0]["achieved"], "frac": cold[0]["frac"],
+                                                    "avg_launch_us": cold[0]["gpu_us"], "how": cold[0]["shape"]}
     return out
 
 
@@ -434,6 +450,9 @@ def main():
     ap.add_argument("--seqlen", type=int, default=384)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="encoder workload: leave out the per-kernel rows of the other configurations and the "
+                         "instruction-rate microbenchmarks")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain elementwise copy of known size (256 MiB read + 256 MiB written), the "
                          "yardstick FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -580,7 +599,7 @@ def main():
             "peak": PEAK_INT8_OPS / 1e12,
             "unit": "TOP/s",
             "frac": round(mha_ops / t_mha / PEAK_INT8_OPS, 4),
-            "traffic": MHA_TRAFFIC_BYTES if default_workload else None,
+            "traffic": measured_traffic("layer", "attention") if default_workload else None,
             "avg_launch_us": round(t_mha * 1e6, 2),
             "algorithmic_ops_per_launch": mha_ops,
             "hbm_frac": round(wl.mha_bytes() / t_mha / PEAK_HBM, 4),
@@ -592,7 +611,7 @@ def main():
             "peak": PEAK_HBM / 1e9,
             "unit": "GB/s",
             "frac": round(ln_bytes / t_ln / PEAK_HBM, 4),
-            "traffic": LN_TRAFFIC_BYTES if default_workload else None,
+            "traffic": measured_traffic("layer", "skipln") if default_workload else None,
             "avg_launch_us": round(t_ln * 1e6, 2),
             "algorithmic_bytes_per_launch": ln_bytes,
             "cold_cache": {"achieved": round(ln_bytes / t_ln_cold / 1e9, 1), "frac": round(ln_bytes / t_ln_cold / PEAK_HBM, 4),

@@ -203,6 +203,15 @@ __global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* 
     out[blockIdx.x * kThreads + threadIdx.x] = s + __float_as_int(t);
 }
 
+// A kernel that does nothing: what a back-to-back launch of a given grid costs on this box.
+__global__ void empty_kernel(int32_t* out)
+{
+    if (out == nullptr && threadIdx.x == 12345)
+    {
+        __builtin_trap(); // never: keeps the parameter alive
+    }
+}
+
 template <typename Launch>
 float time_launches(Launch launch, int reps)
 {
@@ -254,6 +263,12 @@ MB_API float trtamd_microbench_mfma_i8(int shape, int chains, int blocks, int it
     MB_CASE(0, 1) MB_CASE(0, 2) MB_CASE(0, 4) MB_CASE(0, 8) MB_CASE(1, 1) MB_CASE(1, 2) MB_CASE(1, 4) MB_CASE(1, 8)
 #undef MB_CASE
     return -1.f;
+}
+
+// Milliseconds per launch of an empty kernel of `blocks` workgroups of `threads` threads, back to back.
+MB_API float trtamd_microbench_empty(int blocks, int threads, int32_t* out)
+{
+    return time_launches([&] { hipLaunchKernelGGL(empty_kernel, dim3(blocks), dim3(threads), 0, nullptr, out); }, 200);
 }
 
 // Milliseconds per launch; every wavefront issues iters * 4 steps of (one v_mfma_i32_16x16x64_i8, nv v_fma_f32).

@@ -1,17 +1,19 @@
-"""Per-kernel timings on the benchmark configurations other than the headline one.
+"""Per-kernel timings on the benchmark configurations other than the headline pass, and the on-box instruction rates.
 
-    python -m tensorrt_amd.kernel_bench [--steps N]
+bench.py imports `config_rows` and `microbench` and puts their results into its JSON line (keys `configs` and
+`microbench`); `python -m tensorrt_amd.kernel_bench [--steps N]` prints the same rows as a table.
 
-Prints one line per kernel: average launch time (events around back-to-back launches on the launch
-stream), achieved algorithmic bandwidth or arithmetic rate, and its fraction of the MI355X peak
-(HBM 8 TB/s, dense FP16 MFMA 2.5 PFLOP/s, dense INT8 MFMA 5 POP/s).  Inputs are synthetic and
-seeded, resident in HBM; torch is only the allocator.  bench.py remains the one-line contract; this
-is the table behind the per-kernel figures quoted in the design notes.
+Every row: average launch time (events around back-to-back launches on the launch stream), the algorithmic bytes
+or operations of one launch, the achieved rate and its fraction of the MI355X peak (HBM 8 TB/s, dense FP16 MFMA
+2.5 PFLOP/s, dense INT8 MFMA 5 POP/s), and what torch's CPU kernels need for the same subgraph on this host's cores
+(the stand-in for onnxruntime, which is not installed).  Inputs are synthetic and seeded, resident in HBM; torch is
+only the allocator.
 """
 from __future__ import annotations
 
 import argparse
 import ctypes as C
+import os
 import time
 
 import numpy as np
@@ -19,6 +21,7 @@ import numpy as np
 PEAK_HBM = 8.0e12
 PEAK_F16 = 2.5e15
 PEAK_I8 = 5.0e15
+PEAK_F32_MFMA = 157.3e12
 
 
 def f32_bits(x) -> int:
@@ -30,17 +33,85 @@ def half2_bits(x) -> int:
     return h | (h << 16)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--seed", type=int, default=1)
-    args = ap.parse_args()
+def _microbench_lib():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libtrtamd_microbench.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run `python -m tensorrt_amd.build`")
+    lib = C.CDLL(path)
+    lib.trtamd_microbench_mfma_i8.restype = C.c_float
+    lib.trtamd_microbench_mfma_i8.argtypes = [C.c_int] * 4 + [C.c_void_p] * 2
+    lib.trtamd_microbench_valu.restype = C.c_float
+    lib.trtamd_microbench_valu.argtypes = [C.c_int] * 3 + [C.c_void_p] * 3
+    lib.trtamd_microbench_mfma_valu.restype = C.c_float
+    lib.trtamd_microbench_mfma_valu.argtypes = [C.c_int] * 3 + [C.c_void_p] * 2
+    lib.trtamd_microbench_empty.restype = C.c_float
+    lib.trtamd_microbench_empty.argtypes = [C.c_int] * 2 + [C.c_void_p]
+    return lib
 
-    import torch
+
+def microbench(torch, cus: int = 256) -> dict:
+    """Instruction rates of this GPU (csrc/bench/microbench.hip): INT8 MFMA with four independent accumulators per
+    wavefront and four wavefronts per SIMD, on zero and on random operands; the vector-ALU instructions of the softmax;
+    whether the matrix pipe runs beside the vector ALU; the cost of an empty launch."""
+    lib = _microbench_lib()
+    out = torch.zeros(cus * 8 * 256, dtype=torch.int32, device="cuda")
+    zero = torch.zeros(512, dtype=torch.int32, device="cuda")
+    rnd = torch.randint(-2 ** 31, 2 ** 31 - 1, (512,), dtype=torch.int32, device="cuda")
+    clocks = torch.zeros(2 * cus * 8, dtype=torch.int64, device="cuda")
+    wps, chains, iters = 4, 4, 8192
+    blocks = cus * wps
+    res = {"waves_per_simd": wps, "independent_accumulators": chains}
+    # integer operations per instruction and wavefront: 16x16x64 -> 2*16*16*64, 32x32x32 -> 2*32*32*32
+    for shape, name, ops in ((0, "v_mfma_i32_16x16x64_i8", 2 * 16 * 16 * 64), (1, "v_mfma_i32_32x32x32_i8", 2 * 32 * 32 * 32)):
+        for data, dn in ((zero, "zero_operands"), (rnd, "random_operands")):
+            ms = lib.trtamd_microbench_mfma_i8(shape, chains, blocks, iters, data.data_ptr(), out.data_ptr())
+            res[f"{name}.{dn}.TOP/s"] = round(blocks * 4 * iters * chains * ops / (ms * 1e-3) / 1e12, 1)
+    names = ["v_fma_f32", "v_exp_f32", "v_add_f32", "v_perm_b32", "v_max3_i32", "v_cvt_pk_u8_f32",
+             "fma+exp+add+fma (softmax inner sequence)"]
+    valu = {}
+    mhz = []
+    for op, name in enumerate(names):
+        ms = lib.trtamd_microbench_valu(op, blocks, iters, rnd.data_ptr(), out.data_ptr(), clocks.data_ptr())
+        c = clocks[: 2 * blocks].view(blocks, 2).double().cpu().numpy()
+        mhz.append(float((c[:, 0] / np.maximum(c[:, 1], 1)).mean() * 100))
+        valu[name] = ms * 1e-3 / (iters * 8 * wps)          # seconds per wavefront instruction (group) and SIMD
+    clock = float(np.median(mhz)) * 1e6
+    res["shader_clock_MHz_under_vector_load"] = round(clock / 1e6)
+    res["cycles_per_wave_instruction"] = {k: round(v * clock, 2) for k, v in valu.items()}
+    co = {}
+    for nv in (0, 4, 8, 12):
+        ms = lib.trtamd_microbench_mfma_valu(nv, blocks, iters, rnd.data_ptr(), out.data_ptr())
+        co[f"mfma_16x16x64+{nv}_fma"] = round(ms * 1e-3 / (iters * 4 * wps) * clock, 1)
+    res["cycles_per_step_mfma_beside_valu"] = co
+    res["empty_launch_us"] = {f"{b}x{t}": round(lib.trtamd_microbench_empty(b, t, out.data_ptr()) * 1e3, 2)
+                              for b, t in ((256, 256), (1041, 512), (2048, 256))}
+    return res
+
+
+def _cpu_time(fn, budget_s=0.4):
+    """Seconds per call of a torch-CPU subgraph (one warm-up call, then as many as fit the budget)."""
+    fn()
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        fn()
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 50:
+            return el / n
+
+
+def config_rows(api, torch, steps: int = 100, seed: int = 1, cpu: bool = True, launch_floor_us: float | None = None) -> list:
+    """The kernels of configs[0..3] (and of the unfused attention path) at their stated sizes.  launch_floor_us: what
+    an empty kernel costs back to back on this box (microbench()["empty_launch_us"]); bandwidth-bound rows then also
+    carry the rate over the time above that floor, which is what the kernel itself decides at these small sizes."""
     from tensorrt_amd import capi, workloads
-    api = capi.api()
     stream = torch.cuda.current_stream().cuda_stream
-    r = np.random.default_rng(args.seed)
+    r = np.random.default_rng(seed)
+    cores = min(len(os.sched_getaffinity(0)), 16)
+    if cpu:
+        torch.set_num_threads(cores)
+    F = torch.nn.functional
 
     def dev(a):
         return torch.from_numpy(np.ascontiguousarray(a)).cuda()
@@ -50,95 +121,113 @@ def main():
             fn()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(args.steps):
+        for _ in range(steps):
             fn()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / args.steps
-
-    # the GPU raises its clocks over the first tens of milliseconds of load
-    warm = torch.randn((4096, 4096), dtype=torch.float16, device="cuda")
-    t_end = time.perf_counter() + 0.3
-    while time.perf_counter() < t_end:
-        torch.mm(warm, warm)
-        torch.cuda.synchronize()
-    del warm
+        return e0.elapsed_time(e1) * 1e-3 / steps
 
     rows = []
 
-    def report(name, t, nbytes=None, ops=None, peak_ops=None):
+    def report(config, kernel, dtype, shape, t, nbytes=None, ops=None, peak_ops=None, cpu_s=None, note=None):
+        row = {"config": config, "kernel": kernel, "dtype": dtype, "shape": shape, "gpu_us": round(t * 1e6, 2)}
         if nbytes is not None:
-            rows.append((name, t * 1e6, f"{nbytes / t / 1e9:8.1f} GB/s", nbytes / t / PEAK_HBM, "hbm"))
+            row.update({"algorithmic_bytes": int(nbytes), "achieved": round(nbytes / t / 1e9, 1), "unit": "GB/s",
+                        "roofline": "HBM 8 TB/s", "frac": round(nbytes / t / PEAK_HBM, 4)})
+            if launch_floor_us is not None and t * 1e6 > launch_floor_us + 0.2:
+                above = t - launch_floor_us * 1e-6
+                row.update({"empty_launch_us": launch_floor_us, "frac_above_empty_launch": round(nbytes / above / PEAK_HBM, 4)})
         else:
-            rows.append((name, t * 1e6, f"{ops / t / 1e12:8.1f} Top/s", ops / t / peak_ops, "mfma"))
+            row.update({"algorithmic_ops": float(ops), "achieved": round(ops / t / 1e12, 2), "unit": "TOP/s",
+                        "roofline": f"MFMA {peak_ops / 1e12:.1f} TOP/s", "frac": round(ops / t / peak_ops, 4)})
+        if cpu_s is not None:
+            row["cpu_ms"] = round(cpu_s * 1e3, 3)
+            row["cpu"] = f"torch-CPU fallback (onnxruntime unavailable), {cores} cores"
+        if note:
+            row["note"] = note
+        rows.append(row)
 
-    # ---- SkipLayerNorm fp32, [8,128,768] (+bias) ------------------------------------------------
+    # ---- C1: SkipLayerNorm fp32, [8,128,768] + bias -------------------------------------------------
     n_rows, ld = 8 * 128, 768
-    x, s = (dev(r.standard_normal((n_rows, ld)).astype(np.float32)) for _ in range(2))
-    g = dev(r.uniform(0.5, 1.5, ld).astype(np.float32))
-    b = dev((0.1 * r.standard_normal(ld)).astype(np.float32))
-    bias = dev((0.02 * r.standard_normal(ld)).astype(np.float32))
+    hx, hs = (r.standard_normal((n_rows, ld)).astype(np.float32) for _ in range(2))
+    hg = r.uniform(0.5, 1.5, ld).astype(np.float32)
+    hb = (0.1 * r.standard_normal(ld)).astype(np.float32)
+    hbias = (0.02 * r.standard_normal(ld)).astype(np.float32)
+    x, s, g, b, bias = dev(hx), dev(hs), dev(hg), dev(hb), dev(hbias)
     o = torch.empty_like(x)
     t = timeit(lambda: api.check(api.skip_layer_norm_fp32(stream, ld, n_rows * ld, x.data_ptr(), s.data_ptr(),
                                                           b.data_ptr(), g.data_ptr(), o.data_ptr(), bias.data_ptr())))
-    report("SkipLN fp32 1024x768", t, nbytes=n_rows * ld * 3 * 4 + 3 * ld * 4)
+    cpu_s = None
+    if cpu:
+        cx, cs, cg, cb, cbias = (torch.from_numpy(a) for a in (hx, hs, hg, hb, hbias))
+        cpu_s = _cpu_time(lambda: F.layer_norm(cx + cs + cbias, (ld,), cg, cb, 1e-12))
+    report("C1", "SkipLN v5 (skipln_rows_kernel)", "fp32", "1024x768", t, nbytes=n_rows * ld * 3 * 4 + 3 * ld * 4,
+           cpu_s=cpu_s)
 
-    # ---- BERT-base EmbLN + SkipLN fp16, B=32 S=128 E=768 ----------------------------------------
+    # ---- C2: BERT-base EmbLN + SkipLN fp16, B=32 S=128 E=768 ---------------------------------------
     S, B, ld, vocab = 128, 32, 768, 30522
-    word = dev((0.02 * r.standard_normal((vocab, ld))).astype(np.float16))
-    pos = dev((0.02 * r.standard_normal((512, ld))).astype(np.float16))
-    tok = dev((0.02 * r.standard_normal((2, ld))).astype(np.float16))
+    hword = (0.02 * r.standard_normal((vocab, ld))).astype(np.float16)
+    hpos = (0.02 * r.standard_normal((512, ld))).astype(np.float16)
+    htok = (0.02 * r.standard_normal((2, ld))).astype(np.float16)
+    word, pos, tok = dev(hword), dev(hpos), dev(htok)
     g32 = dev(r.uniform(0.5, 1.5, ld).astype(np.float32))
     b32 = dev((0.1 * r.standard_normal(ld)).astype(np.float32))
-    ids = dev(r.integers(0, vocab, (S, B)).astype(np.int32))
-    segs = dev(r.integers(0, 2, (S, B)).astype(np.int32))
+    hids = r.integers(0, vocab, (S, B)).astype(np.int32)
+    hsegs = r.integers(0, 2, (S, B)).astype(np.int32)
+    ids, segs = dev(hids), dev(hsegs)
     emb = torch.empty((S * B, ld), dtype=torch.float16, device="cuda")
     t = timeit(lambda: api.check(api.emb_layer_norm_fp16(stream, ld, B, S, ids.data_ptr(), segs.data_ptr(),
                                                          b32.data_ptr(), g32.data_ptr(), word.data_ptr(),
                                                          pos.data_ptr(), tok.data_ptr(), vocab, 2, emb.data_ptr())))
+    cpu_s = None
+    if cpu:
+        cw, cp, ct = (torch.from_numpy(a.astype(np.float32)) for a in (hword, hpos, htok))
+        ci, cseg = torch.from_numpy(hids.astype(np.int64)), torch.from_numpy(hsegs.astype(np.int64))
+        cg32, cb32 = g32.cpu(), b32.cpu()
+        cpu_s = _cpu_time(lambda: F.layer_norm(cw[ci] + ct[cseg] + cp[:S, None, :], (ld,), cg32, cb32, 1e-12))
     # gathered word rows + output + ids; the position/type rows are shared and stay in cache
-    report("EmbLN fp16 B32 S128 E768", t, nbytes=S * B * (2 * ld * 2 + 8) + S * ld * 2 + 2 * ld * 2)
-    lens = r.integers(64, 129, B)
-    mask = dev((np.arange(S)[:, None] < lens[None, :]).astype(np.int32))
-    pm = torch.zeros((B, 512), dtype=torch.int32, device="cuda")
-    t = timeit(lambda: api.check(api.convert_mask(S, B, 2, 2, 1, mask.data_ptr(), pm.data_ptr(), stream)))
-    report("packed mask B32 S128", t, nbytes=S * B * 4 + B * 512 * 4)
+    report("C2", "EmbLN v6 (embln_kernel)", "fp16", "4096x768, vocab 30522", t,
+           nbytes=S * B * (2 * ld * 2 + 8) + S * ld * 2 + 2 * ld * 2, cpu_s=cpu_s)
     n_rows = S * B
-    xs = dev(r.standard_normal((n_rows, ld)).astype(np.float16))
+    hxs = r.standard_normal((n_rows, ld)).astype(np.float16)
+    xs = dev(hxs)
     gh, bh = g32.half(), b32.half()
     biash = dev((0.02 * r.standard_normal(ld)).astype(np.float16))
     oh = torch.empty_like(emb)
     t = timeit(lambda: api.check(api.skip_layer_norm_fp16(stream, ld, n_rows * ld, emb.data_ptr(), xs.data_ptr(),
                                                           bh.data_ptr(), gh.data_ptr(), oh.data_ptr(),
                                                           biash.data_ptr())))
-    report("SkipLN fp16 4096x768", t, nbytes=n_rows * ld * 3 * 2 + 3 * ld * 2)
+    cpu_s = None
+    if cpu:
+        ce, cxs = emb.float().cpu(), torch.from_numpy(hxs.astype(np.float32))
+        cgh, cbh, cbi = gh.float().cpu(), bh.float().cpu(), biash.float().cpu()
+        cpu_s = _cpu_time(lambda: F.layer_norm(ce + cxs + cbi, (ld,), cgh, cbh, 1e-12))
+    report("C2", "SkipLN v5 (skipln_rows_kernel)", "fp16", "4096x768", t, nbytes=n_rows * ld * 3 * 2 + 3 * ld * 2,
+           cpu_s=cpu_s)
+    # the same kernel where the launch itself no longer matters, operands rotating through more than the 256 MB cache
+    n_big, n_sets = 65536, 6
+    sets = [tuple(torch.randn((n_big, ld), dtype=torch.float16, device="cuda") for _ in range(3)) for _ in range(n_sets)]
+    turn = [0]
 
-    # ---- the same kernels at a size where the launch itself no longer matters -------------------
-    n_big = 65536
-    xb = torch.randn((n_big, ld), dtype=torch.float16, device="cuda")
-    sb = torch.randn((n_big, ld), dtype=torch.float16, device="cuda")
-    ob = torch.empty_like(xb)
-    t = timeit(lambda: api.check(api.skip_layer_norm_fp16(stream, ld, n_big * ld, xb.data_ptr(), sb.data_ptr(),
-                                                          bh.data_ptr(), gh.data_ptr(), ob.data_ptr(),
-                                                          biash.data_ptr())))
-    report("SkipLN fp16 65536x768", t, nbytes=n_big * ld * 3 * 2 + 3 * ld * 2)
-    Sb, Bb = 384, 256
-    idsb = dev(r.integers(0, vocab, (Sb, Bb)).astype(np.int32))
-    segsb = dev(r.integers(0, 2, (Sb, Bb)).astype(np.int32))
-    embb = torch.empty((Sb * Bb, ld), dtype=torch.float16, device="cuda")
-    t = timeit(lambda: api.check(api.emb_layer_norm_fp16(stream, ld, Bb, Sb, idsb.data_ptr(), segsb.data_ptr(),
-                                                         b32.data_ptr(), g32.data_ptr(), word.data_ptr(),
-                                                         pos.data_ptr(), tok.data_ptr(), vocab, 2, embb.data_ptr())))
-    report("EmbLN fp16 B256 S384 E768", t, nbytes=Sb * Bb * (2 * ld * 2 + 8) + Sb * ld * 2 + 2 * ld * 2)
-    del xb, sb, ob, embb
+    def skipln16_rotating():
+        xi, si, oi = sets[turn[0] % n_sets]
+        turn[0] += 1
+        api.check(api.skip_layer_norm_fp16(stream, ld, n_big * ld, xi.data_ptr(), si.data_ptr(), bh.data_ptr(),
+                                           gh.data_ptr(), oi.data_ptr(), biash.data_ptr()))
 
-    # ---- fused attention FP16, BERT-base, B=32, var-seqlen ---------------------------------------
+    t = timeit(skipln16_rotating)
+    report("C2 x16 rows", "SkipLN v5 (skipln_rows_kernel)", "fp16", "65536x768, rotating 1.8 GB", t,
+           nbytes=n_big * ld * 3 * 2 + 3 * ld * 2, note="nothing in the last-level cache")
+    del sets
+
+    # ---- C3: fused attention FP16, BERT-base, B=32, var-seqlen (v5) ---------------------------------
     for S in (128, 384):
         B, N, d = 32, 12, 64
         lens = r.integers(S // 2, S + 1, B)
         cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
         T = int(cu[-1])
-        qkv = dev((r.standard_normal((T, 3 * N * d)) / 8).astype(np.float16))
+        hq = (r.standard_normal((T, 3 * N * d)) / 8).astype(np.float16)
+        qkv = dev(hq)
         out = torch.empty((T, N * d), dtype=torch.float16, device="cuda")
         dcu = dev(cu)
         p = capi.FmhaParams()
@@ -148,72 +237,129 @@ def main():
         p.scale_bmm1, p.scale_softmax, p.scale_bmm2 = half2_bits(0.125), half2_bits(1.0), half2_bits(1.0)
         t = timeit(lambda: api.check(api.fused_mha_run(stream, 1, C.byref(p))))
         ops = 4.0 * d * N * float(np.sum(lens.astype(np.float64) ** 2))
-        report(f"fused MHA fp16 B32 S{S} N12", t, ops=ops, peak_ops=PEAK_F16)
+        cpu_s = None
+        if cpu:
+            cq = torch.from_numpy(hq.astype(np.float32)).reshape(T, N, 3, d)
 
-    # ---- BERT-large INT8 layer pieces in the linear layouts ------------------------------------
-    wl = workloads.int8_layer(64, 384, N=16, seed=args.seed)
+            def attn_cpu():
+                for bb in range(B):
+                    lo, hi = int(cu[bb]), int(cu[bb + 1])
+                    q, k, v = (cq[lo:hi, :, i].transpose(0, 1) for i in range(3))
+                    torch.softmax(q @ k.transpose(1, 2) * 0.125, -1) @ v
+            cpu_s = _cpu_time(attn_cpu)
+        report("C3", "QKV-to-context v5 (fmha_f16_prefix_kernel)", "fp16", f"B=32 N=12 S={S}, {T} tokens", t, ops=ops,
+               peak_ops=PEAK_F16, cpu_s=cpu_s)
+
+    # ---- unfused attention (FP32, other head sizes, S > 512): two MFMA GEMMs around a softmax --------
+    for dt, tname, type_id, peak in ((np.float16, "fp16", 1, PEAK_F16), (np.float32, "fp32", 0, PEAK_F32_MFMA)):
+        S, B, N, d = 128, 32, 12, 64
+        hq = (r.standard_normal((S, B, 3 * N * d)) / 8).astype(dt)
+        qkv = dev(hq)
+        out = torch.empty((S, B, N * d), dtype=qkv.dtype, device="cuda")
+        ws = torch.empty((api.unfused_mha_workspace_size(type_id, S, B, N),), dtype=torch.uint8, device="cuda")
+        t = timeit(lambda: api.check(api.unfused_mha(stream, type_id, S, B, N, d, qkv.data_ptr(), 0, out.data_ptr(),
+                                                     ws.data_ptr())))
+        report("C3 shape, unfused path", "QKV-to-context v4 (batched_gemm_kernel x2 + softmax_rows_kernel)", tname,
+               "S=128 B=32 N=12 d=64, all keys", t, ops=4.0 * d * N * B * S * S, peak_ops=peak,
+               note="three launches, S x S scores through memory")
+
+    # ---- C4: BERT-large INT8 layer, B=64, lengths U[192,384] -----------------------------------------
+    wl = workloads.int8_layer(64, 384, N=16, seed=seed)
     T, E, N = wl.T, wl.E, wl.N
-    qkv_lin = np.ascontiguousarray(wl.qkv_tc.reshape(T, 3, N, 64).transpose(0, 2, 1, 3)).reshape(T, 3 * E)
-    dq = dev(qkv_lin)
-    ctx = torch.empty((T, E), dtype=torch.int8, device="cuda")
+    dq = dev(workloads.interleave32(wl.qkv_tc))
+    ctx = torch.empty((T * E,), dtype=torch.int8, device="cuda")
     dcu = dev(wl.cu)
     p = capi.FmhaParams()
     p.qkv_ptr, p.o_ptr, p.cu_seqlens = dq.data_ptr(), ctx.data_ptr(), dcu.data_ptr()
-    p.qkv_stride_in_bytes, p.o_stride_in_bytes = 3 * E, E
+    p.qkv_stride_in_bytes = p.o_stride_in_bytes = T
     p.b, p.h, p.s, p.d = wl.B, N, wl.S, 64
+    p.interleaved = 1
     p.scale_bmm1 = f32_bits(wl.s_qkv * wl.s_qkv * np.float32(0.125))
     p.scale_softmax, p.scale_bmm2 = f32_bits(127.0), f32_bits(wl.dq_probs * wl.s_qkv / np.float32(0.01))
     t = timeit(lambda: api.check(api.fused_mha_run(stream, 2, C.byref(p))))
-    report("fused MHA int8 (linear) B64 S384 N16", t, ops=wl.mha_ops(), peak_ops=PEAK_I8)
-    skip = dev(wl.skip_tc)
-    gam, bet = dev(wl.gamma), dev(wl.beta)
-    outq = torch.empty((T, E), dtype=torch.int8, device="cuda")
-    t = timeit(lambda: api.check(api.skip_layer_norm_dqq(stream, E, T * E, ctx.data_ptr(), skip.data_ptr(),
-                                                         bet.data_ptr(), gam.data_ptr(), outq.data_ptr(), 0,
-                                                         0.01, float(wl.s_skip), 20.0)))
-    report(f"SkipLN int8 linear {T}x1024", t, nbytes=T * E * 3 + 2 * E * 2)
+    cpu_s = None
+    if cpu:
+        nseq = 8
+        cq = torch.from_numpy(wl.qkv_tc[: int(wl.cu[nseq])].astype(np.float32) * float(wl.s_qkv))
 
-    # ---- SkipLayerNorm with nothing in the last-level cache: operands rotate through more than 256 MB -----
-    Tq = 33289
-    n_sets = 12  # 12 x 3 x 34 MB = 1.2 GB
-    sets = [tuple(torch.randint(-127, 128, (32, Tq, 32), dtype=torch.int8, device="cuda") for _ in range(3))
+        def attn8_cpu():
+            for bb in range(nseq):
+                lo, hi = int(wl.cu[bb]), int(wl.cu[bb + 1])
+                q, k, v = (cq[lo:hi, i * E:(i + 1) * E].reshape(hi - lo, N, 64).transpose(0, 1) for i in range(3))
+                torch.softmax(q @ k.transpose(1, 2) * 0.125, -1) @ v
+        cpu_s = _cpu_time(attn8_cpu) * wl.B / nseq
+    report("C4", "QKV-to-context v6 (fmha_i8_prefix_kernel)", "int8", f"B=64 N=16 S=384, {T} tokens, kCHW32", t,
+           ops=wl.mha_ops(), peak_ops=PEAK_I8, cpu_s=cpu_s,
+           note="CPU: the de-quantised FP32 subgraph on 8 sequences, scaled to 64" if cpu else None)
+    skip = dev(workloads.interleave32(wl.skip_tc))
+    gam, bet = dev(wl.gamma), dev(wl.beta)
+    outq = torch.empty((T * E,), dtype=torch.int8, device="cuda")
+    t = timeit(lambda: api.check(api.skipln_interleaved_large_hface(stream, E, T, ctx.data_ptr(), skip.data_ptr(),
+                                                                   bet.data_ptr(), gam.data_ptr(), outq.data_ptr(),
+                                                                   0.01, float(wl.s_skip), 20.0)))
+    cpu_s = None
+    if cpu:
+        ca, cs2 = (torch.randn(T, E) for _ in range(2))
+        cg, cb = torch.from_numpy(wl.gamma.astype(np.float32)), torch.from_numpy(wl.beta.astype(np.float32))
+        cpu_s = _cpu_time(lambda: F.layer_norm(ca + cs2, (E,), cg, cb, 1e-12))
+    report("C4", "SkipLN v7 (skipln_interleaved_kernel)", "int8", f"{T}x1024 kCHW32, same buffers", t,
+           nbytes=T * E * 3 + 2 * E * 2, cpu_s=cpu_s, note="operands resident in the 256 MB last-level cache")
+    n_sets = 12
+    sets = [tuple(torch.randint(-127, 128, (32, T, 32), dtype=torch.int8, device="cuda") for _ in range(3))
             for _ in range(n_sets)]
-    gh1, bh1 = dev(r.uniform(0.5, 1.5, 1024).astype(np.float16)), dev((0.1 * r.standard_normal(1024)).astype(np.float16))
-    turn = [0]
+    turn[0] = 0
 
     def skipln_rotating():
         xi, si, oi = sets[turn[0] % n_sets]
         turn[0] += 1
-        api.check(api.skipln_interleaved_large_hface(stream, 1024, Tq, xi.data_ptr(), si.data_ptr(), bh1.data_ptr(),
-                                                     gh1.data_ptr(), oi.data_ptr(), 0.02, 0.02, 30.0))
+        api.check(api.skipln_interleaved_large_hface(stream, E, T, xi.data_ptr(), si.data_ptr(), bet.data_ptr(),
+                                                     gam.data_ptr(), oi.data_ptr(), 0.02, 0.02, 30.0))
 
     t = timeit(skipln_rotating)
-    report(f"SkipLN int8 kCHW32 {Tq}x1024, rotating 1.2 GB", t, nbytes=Tq * 1024 * 3 + 2 * 1024 * 2)
-    xi, si, oi = sets[0]
-    t = timeit(lambda: api.check(api.skipln_interleaved_large_hface(
-        stream, 1024, Tq, xi.data_ptr(), si.data_ptr(), bh1.data_ptr(), gh1.data_ptr(), oi.data_ptr(), 0.02, 0.02, 30.0)))
-    report(f"SkipLN int8 kCHW32 {Tq}x1024, same buffers", t, nbytes=Tq * 1024 * 3 + 2 * 1024 * 2)
-    del sets, xi, si, oi
-    n_sets = 6  # 6 x 3 x 100 MB
-    sets = [tuple(torch.randn((n_big, ld), dtype=torch.float16, device="cuda") for _ in range(3)) for _ in range(n_sets)]
+    report("C4", "SkipLN v7 (skipln_interleaved_kernel)", "int8", f"{T}x1024 kCHW32, rotating 0.7 GB", t,
+           nbytes=T * E * 3 + 2 * E * 2, note="nothing in the last-level cache")
+    del sets
+    # ---- C5 SkipLN size, cold ---------------------------------------------------------------------
+    Tq = 33289
+    sets = [tuple(torch.randint(-127, 128, (32, Tq, 32), dtype=torch.int8, device="cuda") for _ in range(3))
+            for _ in range(n_sets)]
     turn[0] = 0
 
-    def skipln16_rotating():
+    def skipln_rotating5():
         xi, si, oi = sets[turn[0] % n_sets]
         turn[0] += 1
-        api.check(api.skip_layer_norm_fp16(stream, ld, n_big * ld, xi.data_ptr(), si.data_ptr(), bh.data_ptr(),
-                                           gh.data_ptr(), oi.data_ptr(), biash.data_ptr()))
+        api.check(api.skipln_interleaved_large_hface(stream, E, Tq, xi.data_ptr(), si.data_ptr(), bet.data_ptr(),
+                                                     gam.data_ptr(), oi.data_ptr(), 0.02, 0.02, 30.0))
 
-    t = timeit(skipln16_rotating)
-    report(f"SkipLN fp16 {n_big}x768, rotating 1.8 GB", t, nbytes=n_big * ld * 3 * 2 + 3 * ld * 2)
+    t = timeit(skipln_rotating5)
+    report("C5", "SkipLN v7 (skipln_interleaved_kernel)", "int8", f"{Tq}x1024 kCHW32, rotating 1.2 GB", t,
+           nbytes=Tq * E * 3 + 2 * E * 2, note="nothing in the last-level cache")
     del sets
+    return rows
 
-    # ---- the linear layers and reformats of the BERT-large INT8 encoder, B=128, 33289 tokens -------------
+
+def extra_rows(api, torch, steps: int = 100) -> list:
+    """Linear layers and reformats of the encoders (the table behind the design notes; not part of bench.py's line)."""
+    from tensorrt_amd import capi
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+
+    def timeit(fn):
+        for _ in range(10):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / steps
 
     def qnormal(shape):
         v = torch.randn(shape, device="cuda")
         return torch.clamp(torch.round(v * (127.0 / float(v.abs().max()))), -127, 127).to(torch.int8)
 
+    Tq = 33289
     for name, K, Nn, epi in (("QKV projection", 1024, 3072, capi.LINEAR_AFFINE),
                              ("attention output projection", 1024, 1024, capi.LINEAR_AFFINE),
                              ("feed-forward 1 + GELU", 1024, 4096, capi.LINEAR_GELU),
@@ -228,9 +374,10 @@ def main():
         lp.a_interleaved = lp.w_interleaved = lp.out_interleaved = 1
         lp.epilogue, lp.out_scale = epi, 30.0
         t = timeit(lambda: api.check(api.int8_linear(stream, C.byref(lp))))
-        report(f"INT8 linear {name} {Tq}x{K}x{Nn}", t, ops=2.0 * Tq * K * Nn, peak_ops=PEAK_I8)
+        ops = 2.0 * Tq * K * Nn
+        rows.append({"kernel": f"INT8 linear {name} {Tq}x{K}x{Nn}", "gpu_us": round(t * 1e6, 2),
+                     "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s", "frac": round(ops / t / PEAK_I8, 4)})
         del a8, w8, o8
-    # ---- FP16 linear layers of a BERT-base FP16 encoder, B=128 x S=128 tokens ---------------------------
     Th = 16384
     for name, K, Nn, epi in (("feed-forward 1 + GELU", 768, 3072, capi.LINEAR_GELU),
                              ("feed-forward 2", 3072, 768, capi.LINEAR_AFFINE)):
@@ -243,18 +390,50 @@ def main():
         hp.a, hp.w, hp.alpha, hp.beta, hp.out = ah.data_ptr(), wh.data_ptr(), al.data_ptr(), be.data_ptr(), oh.data_ptr()
         hp.T, hp.K, hp.N, hp.epilogue = Th, K, Nn, epi
         t = timeit(lambda: api.check(api.fp16_linear(stream, C.byref(hp))))
-        report(f"FP16 linear {name} {Th}x{K}x{Nn}", t, ops=2.0 * Th * K * Nn, peak_ops=PEAK_F16)
+        ops = 2.0 * Th * K * Nn
+        rows.append({"kernel": f"FP16 linear {name} {Th}x{K}x{Nn}", "gpu_us": round(t * 1e6, 2),
+                     "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s", "frac": round(ops / t / PEAK_F16, 4)})
         del ah, wh, oh
     xh = torch.randn((Tq, 1024), dtype=torch.float16, device="cuda")
     x8 = torch.empty((32, Tq, 32), dtype=torch.int8, device="cuda")
-    t = timeit(lambda: api.check(api.quantize_fp16_to_interleaved(stream, Tq, 1024, xh.data_ptr(), 0.03, x8.data_ptr())))
-    report(f"quantise fp16 -> kCHW32 int8 {Tq}x1024", t, nbytes=Tq * 1024 * 3)
-    t = timeit(lambda: api.check(api.dequantize_interleaved_to_fp16(stream, Tq, 1024, x8.data_ptr(), 0.03, xh.data_ptr())))
-    report(f"dequantise kCHW32 int8 -> fp16 {Tq}x1024", t, nbytes=Tq * 1024 * 3)
+    for name, fn in (("quantise fp16 -> kCHW32 int8", lambda: api.check(api.quantize_fp16_to_interleaved(
+                          stream, Tq, 1024, xh.data_ptr(), 0.03, x8.data_ptr()))),
+                     ("dequantise kCHW32 int8 -> fp16", lambda: api.check(api.dequantize_interleaved_to_fp16(
+                          stream, Tq, 1024, x8.data_ptr(), 0.03, xh.data_ptr())))):
+        t = timeit(fn)
+        nb = Tq * 1024 * 3
+        rows.append({"kernel": f"{name} {Tq}x1024", "gpu_us": round(t * 1e6, 2), "achieved": round(nb / t / 1e9, 1),
+                     "unit": "GB/s", "frac": round(nb / t / PEAK_HBM, 4)})
+    return rows
 
-    print(f"{'kernel':52s} {'us':>9s} {'achieved':>16s} {'of peak':>8s}  bound")
-    for name, us, ach, frac, bound in rows:
-        print(f"{name:52s} {us:9.2f} {ach:>16s} {frac:8.3f}  {bound}")
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+
+    import torch
+    from tensorrt_amd import capi
+    api = capi.api()
+    # the GPU raises its clocks over the first tens of milliseconds of load
+    warm = torch.randn((4096, 4096), dtype=torch.float16, device="cuda")
+    t_end = time.perf_counter() + 0.3
+    while time.perf_counter() < t_end:
+        torch.mm(warm, warm)
+        torch.cuda.synchronize()
+    del warm
+    print(f"{'config':22s} {'kernel':62s} {'shape':44s} {'us':>9s} {'achieved':>14s} {'of peak':>8s} {'CPU ms':>9s}")
+    mb = microbench(torch)
+    for row in config_rows(api, torch, args.steps, args.seed, cpu=not args.no_cpu,
+                           launch_floor_us=mb["empty_launch_us"]["256x256"]):
+        print(f"{row['config']:22s} {row['kernel']:62s} {row['shape']:44s} {row['gpu_us']:9.2f} "
+              f"{row['achieved']:9.1f} {row['unit']:>5s} {row['frac']:8.3f} {row.get('cpu_ms', float('nan')):9.2f}")
+    for row in extra_rows(api, torch, args.steps):
+        print(f"{'':22s} {row['kernel']:107s} {row['gpu_us']:9.2f} {row['achieved']:9.1f} {row['unit']:>5s} {row['frac']:8.3f}")
+    for k, v in mb.items():
+        print(f"{k}: {v}")
 
 
 if __name__ == "__main__":
