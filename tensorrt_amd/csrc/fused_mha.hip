@@ -660,17 +660,26 @@ __device__ inline SeqInfo pick_sequence_info(FmhaArgs const& a, int rank, int ca
         atomicAdd(&l.hist[len_bucket(l.cu[t + 1] - l.cu[t])], 1);
     }
     __syncthreads();
-    // bucket that holds position `rank` (longest bucket first) and the offset inside it
-    int k = kLenBuckets - 1;
-    int off = rank;
-    for (; k > 0; --k)
+    // bucket that holds position `rank` (longest bucket first) and the offset inside it: lane k of every wavefront
+    // takes bucket k, a prefix sum over the lanes gives the number of sequences in longer buckets, and the bucket is
+    // the first one with no more than `rank` sequences above it (one LDS read and a few cross-lane steps instead of
+    // a chain of dependent reads, one per bucket)
+    int k, off;
     {
-        int const c = l.hist[k];
-        if (off < c)
+        int const lane = threadIdx.x & (kWaveSize - 1);
+        int const mine = lane < kLenBuckets ? l.hist[lane] : 0;
+        int incl = mine;
+#pragma unroll
+        for (int d = 1; d < kWaveSize; d *= 2)
         {
-            break;
+            int const up = __shfl_up(incl, d);
+            incl += lane >= d ? up : 0;
         }
-        off -= c;
+        int const total = __builtin_amdgcn_readlane(incl, kWaveSize - 1);
+        int const above = total - incl; // sequences in buckets longer than this lane's
+        uint64_t const fits = __ballot(lane < kLenBuckets && above <= rank);
+        k = fits ? (int) __builtin_ctzll(fits) : 0;
+        off = rank - __builtin_amdgcn_readlane(above, k);
     }
     // the off-th sequence (by index) of bucket k: every wavefront scans on its own
     int b = a.B - 1;
@@ -718,6 +727,11 @@ __device__ inline void stage_kv_prefix_i8(FmhaArgs const& a, int64_t seqBase, in
     uint8_t const* src = static_cast<uint8_t const*>(a.qkv);
     int const chunk = threadIdx.x & 3;
     int const rowInPass = threadIdx.x >> 2;
+    // one address per matrix for this lane's first row; every further row of the lane is a whole number of tokens
+    // further on (the address arithmetic of a layout is done once, not once per load)
+    uint8_t const* kSrc = src + qkv_chunk_offset<1, INTERLEAVED>(a, seqBase, firstTok, rowInPass, n, 1, chunk);
+    uint8_t const* vSrc = src + qkv_chunk_offset<1, INTERLEAVED>(a, seqBase, firstTok, rowInPass, n, 2, chunk);
+    int64_t const tokBytes = INTERLEAVED ? 32 : a.tokStrideIn;
     u32x4 kv[KT][kPasses], vv[KT][kPasses];
 #pragma unroll
     for (int kb = 0; kb < KT; ++kb)
@@ -730,13 +744,13 @@ __device__ inline void stage_kv_prefix_i8(FmhaArgs const& a, int64_t seqBase, in
             vv[kb][p] = u32x4{0, 0, 0, 0};
             if (key < nk)
             {
-                kv[kb][p] = *reinterpret_cast<u32x4 const*>(
-                    src + qkv_chunk_offset<1, INTERLEAVED>(a, seqBase, firstTok, key, n, 1, chunk));
-                vv[kb][p] = *reinterpret_cast<u32x4 const*>(
-                    src + qkv_chunk_offset<1, INTERLEAVED>(a, seqBase, firstTok, key, n, 2, chunk));
+                int64_t const step = (int64_t) (kb * 64 + p * kRowsPerPass) * tokBytes;
+                kv[kb][p] = *reinterpret_cast<u32x4 const*>(kSrc + step);
+                vv[kb][p] = *reinterpret_cast<u32x4 const*>(vSrc + step);
             }
         }
     }
+    // LDS positions: a block is 64 rows further on; the swizzle depends on the row inside the block only
 #pragma unroll
     for (int kb = 0; kb < KT; ++kb)
     {
@@ -746,10 +760,9 @@ __device__ inline void stage_kv_prefix_i8(FmhaArgs const& a, int64_t seqBase, in
             for (int p = 0; p < kPasses; ++p)
             {
                 int const kk = p * kRowsPerPass + rowInPass;
-                int const kr = kb * 64 + kk;
-                int const vr = kb * 64 + v_row<1>(kk);
-                *reinterpret_cast<u32x4*>(sK + kr * kRow + swz<1>(kr, chunk) * 16) = kv[kb][p];
-                *reinterpret_cast<u32x4*>(sV + vr * kRow + swz<1>(vr, chunk) * 16) = vv[kb][p];
+                int const vk = v_row<1>(kk);
+                *reinterpret_cast<u32x4*>(sK + kb * 64 * kRow + kk * kRow + swz<1>(kk, chunk) * 16) = kv[kb][p];
+                *reinterpret_cast<u32x4*>(sV + kb * 64 * kRow + vk * kRow + swz<1>(vk, chunk) * 16) = vv[kb][p];
             }
         }
     }
