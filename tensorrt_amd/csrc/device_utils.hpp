@@ -267,6 +267,19 @@ __device__ __forceinline__ void load_to_lds16(void const* g, uint32_t ldsAddr)
     uint32_t const uniform = (uint32_t) __builtin_amdgcn_readfirstlane((int) ldsAddr);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(uniform) : "memory", "m0");
 }
+
+// The same with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit lane offset, the
+// form in which advancing the base from one load to the next is scalar arithmetic and costs the vector ALU nothing.
+__device__ __forceinline__ void load_to_lds16_sbase(void const* base, uint32_t laneOffset, uint32_t ldsAddr)
+{
+    uint64_t const b = reinterpret_cast<uint64_t>(base);
+    uint32_t const lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) b);
+    uint32_t const hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (b >> 32));
+    uint64_t const ub = ((uint64_t) hi << 32) | lo;
+    uint32_t const uniform = (uint32_t) __builtin_amdgcn_readfirstlane((int) ldsAddr);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(laneOffset), "s"(ub), "s"(uniform)
+                 : "memory", "m0");
+}
 #pragma clang diagnostic pop
 
 // s_waitcnt vmcnt(N) alone (the other counters at their maxima): gfx9 encoding, vmcnt in bits 3:0 and 15:14

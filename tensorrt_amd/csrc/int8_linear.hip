@@ -660,32 +660,38 @@ __device__ __forceinline__ void linear_tile_run_dma(
     uint32_t const ldsBase = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lds;
     uint32_t const scaleBase = (uint32_t) (size_t) (__attribute__((address_space(3))) float*) sScale;
 
-    // lane i of a unit's load supplies LDS offset 16 i of the unit
-    auto unit_offset = [&](int u, int row0, int R) -> uint32_t {
+    // Lane i of a unit's load supplies LDS offset 16 i of the unit.  Its address is a wave-uniform part (the unit's
+    // first row, kept in scalar registers and advanced by scalar arithmetic) plus a lane part that is the same for
+    // every unit, tile and stage: the loop spends no vector-ALU instruction on addresses.
+    uint32_t laneOff;
+    if constexpr (IL)
+    {
+        int const r = lane >> 1; // row of the fragment; the half that the swizzle puts at this offset
+        uint32_t const half = (uint32_t) ((lane & 1) ^ ((r >> 3) & 1));
+        laneOff = (uint32_t) r * 32u + half * 16u;
+    }
+    else
+    {
+        int const rr = lane >> 2; // row of the 16-row unit; the chunk that the swizzle puts at this offset
+        uint32_t const chunk = (uint32_t) ((lane & 3) ^ (rr >> 2));
+        laneOff = (uint32_t) rr * (uint32_t) p.K + chunk * 16u;
+    }
+    auto unit_base = [&](int u, int row0, int R) -> uint32_t {
         int const rb = u >> 1, sel = u & 1;
-        if constexpr (IL)
-        {
-            int const r = lane >> 1; // row of the fragment; the half that the swizzle puts at this offset
-            uint32_t const half = (uint32_t) ((lane & 1) ^ ((r >> 3) & 1));
-            return ((uint32_t) sel * (uint32_t) R + (uint32_t) (row0 + rb * 32 + r)) * 32u + half * 16u;
-        }
-        else
-        {
-            int const rr = lane >> 2; // row of the 16-row unit; the chunk that the swizzle puts at this offset
-            uint32_t const chunk = (uint32_t) ((lane & 3) ^ (rr >> 2));
-            return (uint32_t) (row0 + rb * 32 + sel * 16 + rr) * (uint32_t) p.K + chunk * 16u;
-        }
+        uint32_t const b = IL ? ((uint32_t) sel * (uint32_t) R + (uint32_t) (row0 + rb * 32)) * 32u
+                              : (uint32_t) (row0 + rb * 32 + sel * 16) * (uint32_t) p.K;
+        return (uint32_t) __builtin_amdgcn_readfirstlane((int) b);
     };
     auto address = [&](int n0, int t0, uint32_t(&oa)[LA], uint32_t(&ob)[LB]) {
 #pragma unroll
         for (int q = 0; q < LA; ++q)
         {
-            oa[q] = unit_offset(q * NWAVES + wave, n0, p.N);
+            oa[q] = unit_base(q * NWAVES + wave, n0, p.N);
         }
 #pragma unroll
         for (int q = 0; q < LB; ++q)
         {
-            ob[q] = unit_offset(q * NWAVES + wave, t0, p.T);
+            ob[q] = unit_base(q * NWAVES + wave, t0, p.T);
         }
     };
     uint32_t const stepA = IL ? 2u * (uint32_t) p.N * 32u : 64u;
@@ -701,12 +707,14 @@ __device__ __forceinline__ void linear_tile_run_dma(
 #pragma unroll
         for (int q = 0; q < LA; ++q)
         {
-            load_to_lds16(p.w + (next ? oaN[q] : oaC[q]) + k * stepA, dst + (uint32_t) (q * NWAVES + wave) * 1024u);
+            load_to_lds16_sbase(p.w + (uint64_t) (next ? oaN[q] : oaC[q]) + (uint64_t) k * stepA, laneOff,
+                dst + (uint32_t) (q * NWAVES + wave) * 1024u);
         }
 #pragma unroll
         for (int q = 0; q < LB; ++q)
         {
-            load_to_lds16(p.a + (next ? obN[q] : obC[q]) + k * stepB, dst + (uint32_t) (AF + q * NWAVES + wave) * 1024u);
+            load_to_lds16_sbase(p.a + (uint64_t) (next ? obN[q] : obC[q]) + (uint64_t) k * stepB, laneOff,
+                dst + (uint32_t) (AF + q * NWAVES + wave) * 1024u);
         }
     };
 
