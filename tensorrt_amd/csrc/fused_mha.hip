@@ -93,6 +93,7 @@ struct FmhaArgs
     int32_t clampP;              // scale_softmax may push p beyond 127
     int32_t* dbgAcc1;            // optional [B][N][S][S] int32 (INT8) / float bits (FP16)
     int8_t* dbgP8;               // optional [B][N][S][S]
+    int32_t ranked;              // serve the longest sequences first (pointless when one round holds every workgroup)
 };
 
 template <int ESIZE>
@@ -641,9 +642,9 @@ __device__ inline int len_bucket(int len)
 template <int THREADS>
 __device__ inline SeqInfo pick_sequence_info(FmhaArgs const& a, int rank, int capacity, PickLds& l, int& bOut)
 {
-    if (a.cuSeqlens == nullptr || a.B > kMaxRanked)
+    if (a.cuSeqlens == nullptr || a.B > kMaxRanked || !a.ranked)
     {
-        bOut = rank; // fixed layout (equal lengths) or too many sequences: natural order
+        bOut = rank; // fixed layout (equal lengths), too many sequences, or a launch of a single round: natural order
         return seq_info(a, rank, capacity);
     }
     if (threadIdx.x < kLenBuckets)
@@ -1855,6 +1856,15 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
     }
     a.dbgAcc1 = dbgAcc1;
     a.dbgP8 = dbgP8;
+    {
+        // The order in which sequences are served matters when workgroups run in several rounds (the long ones
+        // first, so that the short ones fill the tail).  When every workgroup of the launch is resident at once it
+        // changes nothing, and the workgroups skip the ranking (a trip to LDS and two barriers before their loads).
+        int const kt = pick_kt(p->s);
+        int64_t const lds = dataType == 2 ? Lds<1>::total(kt) : Lds<2>::total(kt);
+        int64_t const perCu = std::max<int64_t>(1, std::min<int64_t>(dataType == 2 ? 3 : 2, (160 * 1024) / std::max<int64_t>(lds, 1)));
+        a.ranked = (int64_t) a.B * a.N * a.qSplit > perCu * 256 ? 1 : 0;
+    }
     if (interleaved)
     {
         // strides carry the total token count (qkvToContextInt8InterleavedPlugin.cpp:280-281)

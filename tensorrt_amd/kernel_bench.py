@@ -66,6 +66,10 @@ def microbench(torch, cus: int = 256) -> dict:
         for data, dn in ((zero, "zero_operands"), (rnd, "random_operands")):
             ms = lib.trtamd_microbench_mfma_i8(shape, chains, blocks, iters, data.data_ptr(), out.data_ptr())
             res[f"{name}.{dn}.TOP/s"] = round(blocks * 4 * iters * chains * ops / (ms * 1e-3) / 1e12, 1)
+    # a dependent chain: one wavefront per SIMD with a single accumulator (each MFMA waits for the one before it)
+    ms = lib.trtamd_microbench_mfma_i8(0, 1, cus, iters, zero.data_ptr(), out.data_ptr())
+    res["v_mfma_i32_16x16x64_i8.one_wave_per_simd_one_accumulator.TOP/s"] = round(
+        cus * 4 * iters * 2 * 16 * 16 * 64 / (ms * 1e-3) / 1e12, 1)
     names = ["v_fma_f32", "v_exp_f32", "v_add_f32", "v_perm_b32", "v_max3_i32", "v_cvt_pk_u8_f32",
              "fma+exp+add+fma (softmax inner sequence)"]
     valu = {}
@@ -78,6 +82,11 @@ def microbench(torch, cus: int = 256) -> dict:
     clock = float(np.median(mhz)) * 1e6
     res["shader_clock_MHz_under_vector_load"] = round(clock / 1e6)
     res["cycles_per_wave_instruction"] = {k: round(v * clock, 2) for k, v in valu.items()}
+    alone = {}
+    for op in (0, 1):
+        ms = lib.trtamd_microbench_valu(op, cus, iters, rnd.data_ptr(), out.data_ptr(), clocks.data_ptr())
+        alone[names[op]] = round(ms * 1e-3 / (iters * 8) * clock, 2)
+    res["cycles_per_wave_instruction_one_wave_per_simd"] = alone
     co = {}
     for nv in (0, 4, 8, 12):
         ms = lib.trtamd_microbench_mfma_valu(nv, blocks, iters, rnd.data_ptr(), out.data_ptr())
