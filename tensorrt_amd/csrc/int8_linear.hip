@@ -2,9 +2,10 @@
 //
 // The projections between the encoder plugins (QKV, attention output, the two feed-forward
 // layers) are plain GEMMs whose operands are both contiguous along k, which is what the INT8 MFMA
-// wants: a lane feeds 16 consecutive k-bytes of one row.  v_mfma_i32_32x32x32_i8 is used because it
-// runs at the full INT8 rate of the matrix core (measured: 32768 MACs in 33 cycles per SIMD);
-// v_mfma_i32_16x16x64_i8 takes 32 cycles for half as many.  The kernel computes the transposed
+// wants: a lane feeds 16 consecutive k-bytes of one row.  v_mfma_i32_32x32x32_i8 is used: it runs at
+// the full INT8 rate of the matrix core (measured: 32768 MACs in 33 cycles per SIMD, as does
+// v_mfma_i32_16x16x64_i8 with 16384 in 16.5) and needs half as many fragment reads per MAC as the
+// 16 x 16 form.  The kernel computes the transposed
 // product (output channels are the M dimension, tokens the N dimension) so that a lane ends up with
 // groups of four consecutive channels of one token, which pack into the token-major INT8 output of
 // either layout.

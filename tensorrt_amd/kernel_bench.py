@@ -126,8 +126,12 @@ def config_rows(api, torch, steps: int = 100, seed: int = 1, cpu: bool = True, l
         return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
     def timeit(fn):
-        for _ in range(10):
-            fn()
+        # the GPU raises its clocks over the first tens of milliseconds of load: 0.15 s of untimed launches first
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.15:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(steps):
@@ -354,8 +358,12 @@ def extra_rows(api, torch, steps: int = 100) -> list:
     rows = []
 
     def timeit(fn):
-        for _ in range(10):
-            fn()
+        # the GPU raises its clocks over the first tens of milliseconds of load: 0.15 s of untimed launches first
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.15:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(steps):
