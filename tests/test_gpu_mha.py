@@ -257,6 +257,32 @@ def test_fmha_packing_invariance_and_special_cases(api):
     assert_fp_close(full[lo:hi], np.broadcast_to(avg, (hi - lo, N * D)), what="uniform attention")
 
 
+def test_fmha_more_sequences_than_the_ranking_holds(api):
+    """Launches of more than 1024 sequences are served in natural order (the longest-first table has 1024 entries);
+    INT8 through the strict decomposition, FP16 against the oracle, and the ranked and unranked orders must agree."""
+    from tensorrt_amd import capi
+    r = rng(27)
+    B, N, S = 1100, 1, 64
+    lens = r.integers(0, S + 1, B)
+    cu = _cu(lens)
+    T = int(cu[-1])
+    qkv, s_q = quantize_amax(r.standard_normal((T, 3 * N * D)))
+    s1 = np.float32(s_q * s_q * np.float32(0.125))
+    got = int8_attention_parity(qkv, cu, N, s1, np.float32(127), np.float32(s_q / (127 * 0.02)), False, S=S)
+    # the first 1000 sequences alone take the ranked path (1000 x 1 workgroups are more than one round): same bytes
+    head = int8_attention_parity(qkv[:cu[1000]].copy(), cu[:1001].copy(), N, s1, np.float32(127),
+                                 np.float32(s_q / (127 * 0.02)), False, S=S)
+    assert np.array_equal(head, got[:cu[1000]])
+    x = (r.standard_normal((T, 3 * N * D)) / 8).astype(np.float16)
+    d_x, d_cu = dev(x), dev(cu)
+    out = dev_empty((T, N * D), np.float16, fill=0)
+    p = _params(capi, qkv_ptr=ptr(d_x), o_ptr=ptr(out), b=B, h=N, s=S, d=D, qkv_stride_in_bytes=2 * 3 * N * D,
+                o_stride_in_bytes=2 * N * D, scale_bmm1=half2_bits(0.125), cu_seqlens=ptr(d_cu))
+    api.check(api.fused_mha_run(stream(), 1, C.byref(p)))
+    sync()
+    assert_fp_close(host(out), oracle.mha_fused_f16_packed(x, cu, N, D), what="FP16, 1100 sequences")
+
+
 def test_fmha_argument_errors(api):
     from tensorrt_amd import capi
     p = _params(capi, qkv_ptr=16, o_ptr=16, b=1, h=1, s=128, d=32, qkv_stride_in_bytes=96, o_stride_in_bytes=32)
