@@ -149,40 +149,50 @@ __device__ inline int64_t qkv_chunk_offset(
     return seqBase + (int64_t) tok * a.tokStrideIn + ((int64_t) n * 3 + mat) * kHeadSize * ESIZE + chunk * 16;
 }
 
-// Builds the 512-bit key-valid mask of sequence b in LDS (sMask[16]).
+// Builds the 512-bit key-valid mask of sequence b in LDS (sMask[16]): every thread takes one key (and one word of the
+// packed mask, if there is one), a wavefront's 64 answers become two words of the mask.
 __device__ inline void build_key_mask(FmhaArgs const& a, int b, int nk, uint32_t* sMask)
 {
-    if (threadIdx.x < 16)
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    for (int key = threadIdx.x; key < 512; key += blockDim.x)
     {
-        uint32_t w = 0;
-        int const k0 = threadIdx.x * 32;
-        if (a.packedMask == nullptr)
-        {
-            int const v = nk - k0;
-            w = v >= 32 ? 0xffffffffu : (v <= 0 ? 0u : ((1u << v) - 1u));
-        }
-        else
+        bool valid = key < nk;
+        if (valid && a.packedMask != nullptr)
         {
             // bit layout of fillSBSMaskKernel (plugin/embLayerNormPlugin/embLayerNormKernel.cu:41-85)
             uint32_t const* pm = a.packedMask + (int64_t) b * a.maskStrideWords;
-            for (int i = 0; i < 32; ++i)
-            {
-                int const key = k0 + i;
-                if (key < nk)
-                {
-                    int const span = 16 * a.warpsN;
-                    int const ni = key / span;
-                    int const r = key % span;
-                    int const warpN = r >> 4;
-                    int const r2 = r & 15;
-                    int const tidx = warpN * a.warpsM * 32 + ((r2 & 7) >> 1);
-                    int const bit = 8 * ni + (r2 & 1) + ((r2 & 8) ? 4 : 0);
-                    w |= ((pm[tidx] >> bit) & 1u) << i;
-                }
-            }
+            int const span = 16 * a.warpsN;
+            int const ni = key / span;
+            int const r = key % span;
+            int const warpN = r >> 4;
+            int const r2 = r & 15;
+            int const tidx = warpN * a.warpsM * 32 + ((r2 & 7) >> 1);
+            int const bit = 8 * ni + (r2 & 1) + ((r2 & 8) ? 4 : 0);
+            valid = ((pm[tidx] >> bit) & 1u) != 0;
         }
-        sMask[threadIdx.x] = w;
+        uint64_t const m = __ballot(valid);
+        if (lane == 0)
+        {
+            sMask[key >> 5] = (uint32_t) m;
+            sMask[(key >> 5) + 1] = (uint32_t) (m >> 32);
+        }
     }
+}
+
+// One past the last key of the mask that takes part (0: none does).  Keys behind it have probability zero whatever
+// their scores, so the kernels treat the sequence as that much shorter: whole blocks of masked keys at the end are
+// neither loaded nor multiplied.  sMask must be complete (barrier) before the call; the result is wave-uniform.
+__device__ inline int used_keys(uint32_t const* sMask, int nk)
+{
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    uint32_t const w = lane < 16 ? sMask[lane] : 0u;
+    int end = w ? lane * 32 + 32 - __builtin_clz(w) : 0;
+#pragma unroll
+    for (int d = 1; d < 16; d *= 2)
+    {
+        end = max(end, __shfl_xor(end, d));
+    }
+    return min(__builtin_amdgcn_readfirstlane(end), nk);
 }
 
 // Stage K and V of one (sequence, head) into LDS, 16 bytes per lane per access.  Rows at or
@@ -353,11 +363,12 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
     {
         return; // no query tile for this workgroup
     }
-    int const nkb = (sq.nk + 63) >> 6;
-    int const ntile = (sq.nk + 15) >> 4; // 16-key tiles that hold at least one key
     build_key_mask(a, b, sq.nk, sMask);
     __syncthreads();
-    stage_kv<1, KT, INTERLEAVED, kWavesI8>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sMask, sK, sV);
+    int const nkUsed = used_keys(sMask, sq.nk);
+    int const nkb = (nkUsed + 63) >> 6;
+    int const ntile = (nkUsed + 15) >> 4; // 16-key tiles that hold at least one key
+    stage_kv<1, KT, INTERLEAVED, kWavesI8>(a, sq.seqBaseIn, sq.firstTok, n, nkUsed, nkb, sMask, sK, sV);
     __syncthreads();
 
     int const lane = threadIdx.x & (kWaveSize - 1);
@@ -429,7 +440,7 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
                         for (int j = 0; j < 4; ++j)
                         {
                             int const key = kb * 64 + u * 16 + g * 4 + j;
-                            if (key < sq.nk)
+                            if (key < nkUsed)
                             {
                                 a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
                                     = acc[kb * 4 + u][j] - kMagicBits;
@@ -558,7 +569,7 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
                         for (int j = 0; j < 4; ++j)
                         {
                             int const key = kb * 64 + u * 16 + g * 4 + j;
-                            if (key < sq.nk)
+                            if (key < nkUsed)
                             {
                                 a.dbgP8[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
                                     = (int8_t) ((uint32_t) preg[u] >> (8 * j));
@@ -1089,10 +1100,11 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
     {
         return;
     }
-    int const nkb = (sq.nk + 63) >> 6;
     build_key_mask(a, b, sq.nk, sMask);
     __syncthreads();
-    stage_kv<2, KT, false, kWavesF16>(a, sq.seqBaseIn, sq.firstTok, n, sq.nk, nkb, sMask, sK, sV);
+    int const nkUsed = used_keys(sMask, sq.nk);
+    int const nkb = (nkUsed + 63) >> 6;
+    stage_kv<2, KT, false, kWavesF16>(a, sq.seqBaseIn, sq.firstTok, n, nkUsed, nkb, sMask, sK, sV);
     __syncthreads();
 
     int const lane = threadIdx.x & (kWaveSize - 1);
@@ -1173,7 +1185,7 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
                         for (int j = 0; j < 4; ++j)
                         {
                             int const key = kb * 64 + u * 16 + g * 4 + j;
-                            if (key < sq.nk)
+                            if (key < nkUsed)
                             {
                                 a.dbgAcc1[(((int64_t) b * a.N + n) * a.S + q) * a.S + key]
                                     = __float_as_int(acc[kb * 4 + u][j]);

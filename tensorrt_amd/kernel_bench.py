@@ -263,6 +263,29 @@ def config_rows(api, torch, steps: int = 100, seed: int = 1, cpu: bool = True, l
         report("C3", "QKV-to-context v5 (fmha_f16_prefix_kernel)", "fp16", f"B=32 N=12 S={S}, {T} tokens", t, ops=ops,
                peak_ops=PEAK_F16, cpu_s=cpu_s)
 
+    # ---- C3, the fixed [S,B,N,3,d] layout with the packed key mask (v4 plugin with a mask input) ----------
+    for S in (128, 384):
+        B, N, d = 32, 12, 64
+        lens = r.integers(S // 2, S + 1, B)
+        hq = (r.standard_normal((S, B, 3 * N * d)) / 8).astype(np.float16)
+        qkv = dev(hq)
+        out = torch.empty((S, B, N * d), dtype=torch.float16, device="cuda")
+        mask = dev((np.arange(S)[:, None] < lens[None, :]).astype(np.int32))
+        words = 6144 if S == 384 else 512
+        packed = torch.zeros((B, words), dtype=torch.int32, device="cuda")
+        wm, wn = (2, 2) if S <= 128 else (1, 8)
+        api.check(api.convert_mask(S, B, wm, wn, 1, mask.data_ptr(), packed.data_ptr(), stream))
+        p = capi.FmhaParams()
+        p.qkv_ptr, p.o_ptr, p.packed_mask_ptr = qkv.data_ptr(), out.data_ptr(), packed.data_ptr()
+        p.qkv_stride_in_bytes, p.o_stride_in_bytes = 3 * B * N * d * 2, B * N * d * 2
+        p.packed_mask_stride_in_bytes = words * 4
+        p.b, p.h, p.s, p.d = B, N, S, d
+        p.scale_bmm1, p.scale_softmax, p.scale_bmm2 = half2_bits(0.125), half2_bits(1.0), half2_bits(1.0)
+        t = timeit(lambda: api.check(api.fused_mha_run(stream, 1, C.byref(p))))
+        report("C3", "QKV-to-context v4, packed mask (fmha_f16_kernel)", "fp16", f"S={S} B=32 N=12, fixed layout", t,
+               ops=4.0 * d * N * float(np.sum(lens.astype(np.float64) ** 2)), peak_ops=PEAK_F16,
+               note="every query row of the S x B tensor is computed; ops count valid lengths only")
+
     # ---- unfused attention (FP32, other head sizes, S > 512): two MFMA GEMMs around a softmax --------
     for dt, tname, type_id, peak in ((np.float16, "fp16", 1, PEAK_F16), (np.float32, "fp32", 0, PEAK_F32_MFMA)):
         S, B, N, d = 128, 32, 12, 64
@@ -304,6 +327,17 @@ def config_rows(api, torch, steps: int = 100, seed: int = 1, cpu: bool = True, l
     report("C4", "QKV-to-context v6 (fmha_i8_prefix_kernel)", "int8", f"B=64 N=16 S=384, {T} tokens, kCHW32", t,
            ops=wl.mha_ops(), peak_ops=PEAK_I8, cpu_s=cpu_s,
            note="CPU: the de-quantised FP32 subgraph on 8 sequences, scaled to 64" if cpu else None)
+    # the same attention in the linear layout of the v5 plugin ([T, 3E], channel order [N][3][d])
+    dql = dev(np.ascontiguousarray(wl.qkv_tc.reshape(T, 3, N, 64).transpose(0, 2, 1, 3)).reshape(T, 3 * E))
+    ctxl = torch.empty((T, E), dtype=torch.int8, device="cuda")
+    pl = capi.FmhaParams()
+    pl.qkv_ptr, pl.o_ptr, pl.cu_seqlens = dql.data_ptr(), ctxl.data_ptr(), dcu.data_ptr()
+    pl.qkv_stride_in_bytes, pl.o_stride_in_bytes = 3 * E, E
+    pl.b, pl.h, pl.s, pl.d = wl.B, N, wl.S, 64
+    pl.scale_bmm1, pl.scale_softmax, pl.scale_bmm2 = p.scale_bmm1, p.scale_softmax, p.scale_bmm2
+    t = timeit(lambda: api.check(api.fused_mha_run(stream, 2, C.byref(pl))))
+    report("C4", "QKV-to-context v5 (fmha_i8_prefix_kernel, linear layout)", "int8",
+           f"B=64 N=16 S=384, {T} tokens, [T,3E]", t, ops=wl.mha_ops(), peak_ops=PEAK_I8)
     skip = dev(workloads.interleave32(wl.skip_tc))
     gam, bet = dev(wl.gamma), dev(wl.beta)
     outq = torch.empty((T * E,), dtype=torch.int8, device="cuda")
