@@ -135,6 +135,100 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(int const ld, int6
     }
 }
 
+// The same for rows that are whole 16-byte pieces at 16-byte aligned addresses: LPR lanes share a row (64 / LPR rows
+// per wavefront), each taking NV pieces of 16 bytes, piece j of a lane LPR pieces behind piece j - 1, so that every
+// access of the wavefront covers whole 64-byte runs and a short row does not leave most of the lanes idle.
+template <typename T, int LPR, int NV>
+__global__ __launch_bounds__(kBlock) void softmax_rows_vec_kernel(int const ld, int64_t const rows,
+    int64_t const rowsPerBatch, float const w, int32_t const* __restrict__ maskIdx, T const* __restrict__ in,
+    T* __restrict__ out)
+{
+    constexpr int V = 16 / sizeof(T);              // elements per piece
+    constexpr int kRowsPerWave = kWaveSize / LPR;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const sub = lane % LPR;
+    int64_t const row
+        = ((int64_t) blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * kRowsPerWave + lane / LPR;
+    bool const live = row < rows;
+    int lastValid = 0;
+    if (live)
+    {
+        lastValid = maskIdx ? min(ld, maskIdx[row / rowsPerBatch]) : ld;
+    }
+    T const* x = in + (live ? row : 0) * ld;
+    float const wl2 = w * 1.4426950408889634f;
+    float v[NV][V];
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+    {
+        int const i0 = (sub + LPR * j) * V;
+        T raw[V];
+        if (live && i0 < ld)
+        {
+            *reinterpret_cast<u32x4*>(raw) = *reinterpret_cast<u32x4 const*>(x + i0);
+        }
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+        {
+            v[j][e] = (live && i0 + e < lastValid) ? (float) raw[e] : -3.0e38f;
+            mx = fmaxf(mx, v[j][e]);
+        }
+    }
+#pragma unroll
+    for (int d = 1; d < LPR; d *= 2)
+    {
+        mx = fmaxf(mx, __shfl_xor(mx, d));
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+    {
+        int const i0 = (sub + LPR * j) * V;
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+        {
+            v[j][e] = i0 + e < lastValid ? __builtin_amdgcn_exp2f((v[j][e] - mx) * wl2) : 0.f;
+            sum += v[j][e];
+        }
+    }
+#pragma unroll
+    for (int d = 1; d < LPR; d *= 2)
+    {
+        sum += __shfl_xor(sum, d);
+    }
+    float const rz = 1.f / sum;
+    if (live)
+    {
+        T* y = out + row * ld;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+        {
+            int const i0 = (sub + LPR * j) * V;
+            if (i0 < ld)
+            {
+                T res[V];
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                {
+                    res[e] = (T) (i0 + e < lastValid ? v[j][e] * rz : 0.f);
+                }
+                *reinterpret_cast<u32x4*>(y + i0) = *reinterpret_cast<u32x4 const*>(res);
+            }
+        }
+    }
+}
+
+template <typename T, int LPR, int NV>
+void launch_softmax_vec(hipStream_t stream, int32_t ld, int64_t rows, int64_t rpb, float w, int32_t const* maskIdx,
+    T const* in, T* out)
+{
+    int64_t const rowsPerBlock = (int64_t) kWavesPerBlock * (kWaveSize / LPR);
+    dim3 const grid((unsigned) ceil_div<int64_t>(rows, rowsPerBlock));
+    hipLaunchKernelGGL((softmax_rows_vec_kernel<T, LPR, NV>), grid, dim3(kBlock), 0, stream, ld, rows, rpb, w, maskIdx, in,
+        out);
+}
+
 template <typename T>
 int scaled_softmax(hipStream_t stream, int32_t ld, int32_t B, int32_t N, float w, int32_t const* maskIdx, T const* in,
     T* out)
@@ -152,8 +246,32 @@ int scaled_softmax(hipStream_t stream, int32_t ld, int32_t B, int32_t N, float w
     {
         return set_error(TRTAMD_STATUS_BAD_PARAM, "scaledSoftmax: null pointer");
     }
-    dim3 const grid((unsigned) ceil_div<int64_t>(rows, kWavesPerBlock));
     int64_t const rpb = (int64_t) N * ld;
+    // rows of whole, aligned 16-byte pieces of up to 512 elements: the vectorised kernel
+    constexpr int V = 16 / (int) sizeof(T);
+    if (ld % V == 0 && ld <= 512 && (reinterpret_cast<uintptr_t>(in) & 15) == 0
+        && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
+    {
+        int const pieces = ld / V;
+        if (pieces <= 16)
+        {
+            launch_softmax_vec<T, 16, 1>(stream, ld, rows, rpb, w, maskIdx, in, out);
+        }
+        else if (pieces <= 32)
+        {
+            launch_softmax_vec<T, 32, 1>(stream, ld, rows, rpb, w, maskIdx, in, out);
+        }
+        else if (pieces <= 64)
+        {
+            launch_softmax_vec<T, 64, 1>(stream, ld, rows, rpb, w, maskIdx, in, out);
+        }
+        else
+        {
+            launch_softmax_vec<T, 64, 2>(stream, ld, rows, rpb, w, maskIdx, in, out);
+        }
+        return check_launch("softmax_rows_vec_kernel");
+    }
+    dim3 const grid((unsigned) ceil_div<int64_t>(rows, kWavesPerBlock));
     if (ld <= 128)
     {
         hipLaunchKernelGGL((softmax_rows_kernel<T, 2>), grid, dim3(kBlock), 0, stream, ld, rows, rpb, w, maskIdx, in, out);
