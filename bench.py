@@ -135,26 +135,49 @@ def run_encoder(args, api, torch):
     got = step()
     torch.cuda.synchronize()
     assert torch.equal(got, want), "native runner and Python chain disagree"
+    single = step
+    streams = 1 if args.python_runner else max(1, args.streams)
+    if streams > 1:
+        # the same batch as `streams` runs of whole sequences that the runner executes at the same time (one
+        # execution context and stream each): the same output bits, and the tail of every kernel of one run is
+        # filled by the other
+        streams = enc.prepare_concurrent(streams)
+        step = lambda: enc.enqueue_native_concurrent(streams)
+        got.zero_()
+        got = step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), "concurrent sub-batches and the single pass disagree"
     if args.graph and not args.python_runner:
         # the native enqueue only launches kernels: record one pass, time its replays
+        eager = step
+        cap_stream = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            got = enc.enqueue_native(stream=torch.cuda.current_stream().cuda_stream)
+        with torch.cuda.stream(cap_stream):
+            with torch.cuda.graph(graph, stream=cap_stream):
+                if streams > 1:
+                    got = enc.enqueue_native_concurrent(streams, stream=cap_stream.cuda_stream)
+                else:
+                    got = enc.enqueue_native(stream=cap_stream.cuda_stream)
         step = graph.replay
         got.zero_()
         step()
         torch.cuda.synchronize()
         assert torch.equal(got, want), "graph replay and eager pass disagree"
 
-    clock_ramp(torch, step)
-    for _ in range(max(args.warmup, 1)):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    def timed(fn, steps, warmup):
+        clock_ramp(torch, fn)
+        for _ in range(max(warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    ms_step = timed(step, args.steps, args.warmup)
+    # the single enqueue on one stream, for the record (a tenth of the steps)
+    ms_single = ms_step if streams == 1 and not args.graph else timed(single, max(args.steps // 10, 5), 3)
 
     # per-kernel durations (layer 0's operations, back-to-back launches between two events)
     b, L = enc.buf, enc.layers[0]
@@ -186,7 +209,7 @@ def run_encoder(args, api, torch):
     ln_bytes = float(T) * E * 3 + 4 * E
     per_layer = sum(times.values()) + times["skipln"]
     table = {k: {"avg_launch_us": round(t * 1e6, 2),
-                 "share_of_pass": round(t * (2 if k == "skipln" else 1) * cfg.layers / (ms_step * 1e-3), 4)}
+                 "share_of_pass": round(t * (2 if k == "skipln" else 1) * cfg.layers / (ms_single * 1e-3), 4)}
              for k, t in times.items()}
     for k, (_, n_ops) in ops.items():
         if n_ops:
@@ -223,9 +246,14 @@ def run_encoder(args, api, torch):
                         "GEMM / SkipLayerNorm v7, dequantise; random-init weights, scales calibrated on the batch",
             "batch": args.batch, "max_seq_len": args.seqlen, "heads": N, "head_size": 64, "hidden": E, "ffn": F,
             "layers": cfg.layers, "tokens": T, "lengths": f"uniform[128,{args.seqlen}] seed {args.seed}",
-            "runner": "python" if args.python_runner else "native (trtamd_encoder_enqueue)"
+            "runner": "python" if args.python_runner else
+                      ("native (trtamd_encoder_enqueue_concurrent)" if streams > 1 else "native (trtamd_encoder_enqueue)")
                       + (", replayed from a captured graph" if args.graph else ""),
+            "parallelism": "one GPU" + (f"; the batch runs as {streams} sub-batches of whole sequences at the same time "
+                                        f"(one execution context and stream each), output bits equal to the single "
+                                        f"enqueue's" if streams > 1 else "; one stream"),
         },
+        "ms_per_step_single_stream": round(ms_single, 4),
         "roofline": {
             "kernel": "int8_linear_dma_kernel<true,GELU> (feed-forward 1)",
             "bound": "mfma",
@@ -444,6 +472,8 @@ def main():
     ap.add_argument("--layers", type=int, default=24, help="encoder workload only")
     ap.add_argument("--graph", action="store_true",
                     help="encoder workload: record the native runner's pass into a graph and time its replays")
+    ap.add_argument("--streams", type=int, default=2,
+                    help="encoder workload: sub-batches of the batch that run at the same time (1: a single enqueue)")
     ap.add_argument("--python-runner", action="store_true",
                     help="encoder workload: time the Python chain of plugin calls instead of the C++ runner")
     ap.add_argument("--batch", type=int, default=None, help="default 64 (layer) / 128 (encoder)")

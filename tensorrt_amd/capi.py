@@ -72,6 +72,12 @@ class EncoderLayer(C.Structure):
                 ("ln1_gamma", c_p), ("ln1_beta", c_p), ("ln2_gamma", c_p), ("ln2_beta", c_p),
                 ("s_x", f32), ("s_qkv", f32), ("s_ctx", f32), ("s_ao", f32), ("s_h", f32), ("s_f", f32), ("s_out", f32)]
 
+
+class EncoderBatch(C.Structure):
+    _fields_ = [("ids", c_p), ("segment_ids", c_p), ("cu_seqlens", c_p), ("batch", i32), ("tokens", i32),
+                ("workspace", c_p), ("out", c_p)]
+
+
 _SIGS = {
     "trtamd_version": (C.c_int, []),
     "trtamd_last_error": (C.c_char_p, []),
@@ -115,6 +121,8 @@ _SIGS = {
     "trtamd_encoder_set_layer": (C.c_int, [c_p, i32, C.POINTER(EncoderLayer)]),
     "trtamd_encoder_workspace_size": (C.c_size_t, [c_p, i32]),
     "trtamd_encoder_enqueue": (C.c_int, [c_p, c_p, c_p, c_p, i32, i32, c_p, c_p, c_p]),
+    "trtamd_encoder_reserve_contexts": (C.c_int, [c_p, i32]),
+    "trtamd_encoder_enqueue_concurrent": (C.c_int, [c_p, C.POINTER(EncoderBatch), i32, c_p]),
     "trtamd_int8_linear_to_interleaved": (C.c_int, [c_p, i32, i32, c_p, c_p]),
     "trtamd_int8_interleaved_to_linear": (C.c_int, [c_p, i32, i32, c_p, c_p]),
     "trtamd_quantize_fp16_to_interleaved": (C.c_int, [c_p, i32, i32, c_p, f32, c_p]),
@@ -129,7 +137,8 @@ ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear", "trtamd_fp16_linear", "trtamd_int8_
                        "trtamd_quantize_fp16_to_interleaved", "trtamd_dequantize_interleaved_to_fp16"]
 # Entry points declared in include/trtamd_encoder_runtime.h.
 ENCODER_RUNTIME_SYMBOLS = ["trtamd_encoder_create", "trtamd_encoder_destroy", "trtamd_encoder_set_embedding",
-                           "trtamd_encoder_set_layer", "trtamd_encoder_workspace_size", "trtamd_encoder_enqueue"]
+                           "trtamd_encoder_set_layer", "trtamd_encoder_workspace_size", "trtamd_encoder_enqueue",
+                           "trtamd_encoder_reserve_contexts", "trtamd_encoder_enqueue_concurrent"]
 HEADER_SYMBOLS = [k for k in _SIGS if k not in TEST_HOOK_SYMBOLS and k not in ENCODER_OPS_SYMBOLS
                   and k not in ENCODER_RUNTIME_SYMBOLS]
 

@@ -111,10 +111,17 @@ struct LinearLayer
     }
 };
 
+// The plugin objects of one layer.  They keep per-shape state between onShapeChange and enqueue, so every execution
+// context has a set of its own (clones of the first one, as TensorRT clones an engine's plugins for each
+// IExecutionContext it creates).
+struct LayerPlugins
+{
+    PluginPtr attention, ln1, ln2;
+};
+
 struct Layer
 {
     LinearLayer qkv, proj, ffn1, ffn2;
-    PluginPtr attention, ln1, ln2;
     float ffn1OutScale{1.f};
     float sX{0}, sQkv{0}, sCtx{0}, sAo{0}, sH{0}, sF{0}, sOut{0};
     bool set{false};
@@ -136,7 +143,12 @@ public:
             "the INT8 interleaved attention plugin serves heads of 64 channels");
         TRTAMD_VALIDATE(c.hidden % 64 == 0 && c.ffn % 64 == 0 && c.ffn > 0 && c.layers >= 0);
         TRTAMD_VALIDATE(c.vocab > 0 && c.max_pos > 0 && c.type_vocab > 0 && c.max_seqlen > 0 && c.max_seqlen <= 512);
+        mContexts.resize(1);
+        mContexts[0].layers.resize(static_cast<size_t>(c.layers));
     }
+
+    Encoder(Encoder const&) = delete;
+    Encoder& operator=(Encoder const&) = delete;
 
     void setEmbedding(trtamd_encoder_embedding const& e)
     {
@@ -150,7 +162,8 @@ public:
             {"bert_embeddings_token_type_embeddings", e.tok, PluginFieldType::kFLOAT32, mCfg.type_vocab * E},
             {"bert_embeddings_position_embeddings", e.pos, PluginFieldType::kFLOAT32, mCfg.max_pos * E},
             {"output_fp16", &fp16, PluginFieldType::kINT32, 1}};
-        mEmbedding = makeRuntimePlugin(kEMB, "4", "embeddings", f);
+        TRTAMD_VALIDATE_MSG(mContexts.size() == 1, "set_embedding after reserve_contexts");
+        mContexts[0].embedding = makeRuntimePlugin(kEMB, "4", "embeddings", f);
         mEmbScale = e.scale;
     }
 
@@ -159,8 +172,10 @@ public:
         TRTAMD_VALIDATE_MSG(index >= 0 && index < mCfg.layers, "layer index out of range");
         TRTAMD_VALIDATE(l.ln1_gamma && l.ln1_beta && l.ln2_gamma && l.ln2_beta);
         TRTAMD_VALIDATE(l.s_x > 0 && l.s_qkv > 0 && l.s_ctx > 0 && l.s_ao > 0 && l.s_h > 0 && l.s_f > 0 && l.s_out > 0);
+        TRTAMD_VALIDATE_MSG(mContexts.size() == 1, "set_layer after reserve_contexts");
         int32_t const E = mCfg.hidden, F = mCfg.ffn;
         Layer& L = mLayers[static_cast<size_t>(index)];
+        LayerPlugins& P = mContexts[0].layers[static_cast<size_t>(index)];
         L.qkv.load(l.qkv, 3 * E, E);
         L.proj.load(l.proj, E, E);
         L.ffn1.load(l.ffn1, F, E);
@@ -170,30 +185,14 @@ public:
         float const dqProbs = 1.f / 127.f;
         std::vector<PluginField> qf{{"hidden_size", &mCfg.hidden, PluginFieldType::kINT32, 1},
             {"num_heads", &mCfg.heads, PluginFieldType::kINT32, 1}, {"dq_probs", &dqProbs, PluginFieldType::kFLOAT32, 1}};
-        L.attention = makeRuntimePlugin(kQKV, "6", tag + "_attention", qf);
+        P.attention = makeRuntimePlugin(kQKV, "6", tag + "_attention", qf);
         auto ln = [&](char const* which, trtamd_half_t const* gamma, trtamd_half_t const* beta) {
             std::vector<PluginField> f{{"beta", beta, PluginFieldType::kFLOAT16, E}, {"gamma", gamma, PluginFieldType::kFLOAT16, E}};
             return makeRuntimePlugin(kSKIP, "7", tag + which, f);
         };
-        L.ln1 = ln("_ln1", l.ln1_gamma, l.ln1_beta);
-        L.ln2 = ln("_ln2", l.ln2_gamma, l.ln2_beta);
-        // One shape change with representative descriptors here, so that whatever a plugin sets up on its first
-        // shape change (device copies of parameters, kernel attributes) is done before the first enqueue, which
-        // a caller may be recording into a graph.
-        {
-            int64_t const T = mCfg.max_seqlen;
-            auto const il = TensorFormat::kCHW32;
-            auto const lin = TensorFormat::kLINEAR;
-            PluginTensorDesc const act = desc({1, E, T, 1}, DataType::kINT8, il, 1.f);
-            PluginTensorDesc const lnIn[2] = {act, act};
-            for (PluginPtr const* p : {&L.ln1, &L.ln2})
-            {
-                TRTAMD_VALIDATE_MSG(runtimeOf(*p)->onShapeChange(lnIn, 2, &act, 1) == 0, tag + ": SkipLayerNorm set-up failed");
-            }
-            PluginTensorDesc const qIn[3] = {desc({1, 3 * E, T, 1}, DataType::kINT8, il, 1.f),
-                desc({2}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f)};
-            TRTAMD_VALIDATE_MSG(runtimeOf(L.attention)->onShapeChange(qIn, 3, &act, 1) == 0, tag + ": attention set-up failed");
-        }
+        P.ln1 = ln("_ln1", l.ln1_gamma, l.ln1_beta);
+        P.ln2 = ln("_ln2", l.ln2_gamma, l.ln2_beta);
+        firstShapeChange(P, tag);
         L.sX = l.s_x;
         L.sQkv = l.s_qkv;
         L.sCtx = l.s_ctx;
@@ -202,6 +201,64 @@ public:
         L.sF = l.s_f;
         L.sOut = l.s_out;
         L.set = true;
+    }
+
+    // One shape change with representative descriptors, so that whatever a plugin sets up on its first shape change
+    // (device copies of parameters, kernel attributes) is done before the first enqueue, which a caller may be
+    // recording into a graph.
+    void firstShapeChange(LayerPlugins const& P, std::string const& tag) const
+    {
+        int64_t const T = mCfg.max_seqlen, E = mCfg.hidden;
+        auto const il = TensorFormat::kCHW32;
+        auto const lin = TensorFormat::kLINEAR;
+        PluginTensorDesc const act = desc({1, E, T, 1}, DataType::kINT8, il, 1.f);
+        PluginTensorDesc const lnIn[2] = {act, act};
+        for (PluginPtr const* p : {&P.ln1, &P.ln2})
+        {
+            TRTAMD_VALIDATE_MSG(runtimeOf(*p)->onShapeChange(lnIn, 2, &act, 1) == 0, tag + ": SkipLayerNorm set-up failed");
+        }
+        PluginTensorDesc const qIn[3] = {desc({1, 3 * E, T, 1}, DataType::kINT8, il, 1.f),
+            desc({2}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f)};
+        TRTAMD_VALIDATE_MSG(runtimeOf(P.attention)->onShapeChange(qIn, 3, &act, 1) == 0, tag + ": attention set-up failed");
+    }
+
+    // Execution contexts beyond the first: clones of every plugin object (IPluginV3::clone, what TensorRT does for
+    // each IExecutionContext of an engine), and for each of them a stream and two events of the runner's own, so
+    // that enqueueConcurrent has nothing left to create.  Weights and scales are shared.
+    void reserveContexts(int32_t count)
+    {
+        TRTAMD_VALIDATE_MSG(count >= 1 && count <= kMaxContexts, "between 1 and 8 execution contexts");
+        requireComplete();
+        while (static_cast<int32_t>(mContexts.size()) < count)
+        {
+            Context c;
+            Context const& first = mContexts[0];
+            auto cloneOf = [](PluginPtr const& p, char const* what) {
+                PluginPtr q(p->clone());
+                TRTAMD_VALIDATE_MSG(q != nullptr, std::string(what) + ": clone failed");
+                return q;
+            };
+            c.embedding = cloneOf(first.embedding, "EmbLayerNorm");
+            c.layers.resize(first.layers.size());
+            for (size_t i = 0; i < first.layers.size(); ++i)
+            {
+                c.layers[i].attention = cloneOf(first.layers[i].attention, "QKV-to-context");
+                c.layers[i].ln1 = cloneOf(first.layers[i].ln1, "SkipLayerNorm 1");
+                c.layers[i].ln2 = cloneOf(first.layers[i].ln2, "SkipLayerNorm 2");
+                firstShapeChange(c.layers[i], "context " + std::to_string(mContexts.size()) + " l" + std::to_string(i));
+            }
+            // default priority, no implicit synchronisation with the null stream
+            TRTAMD_VALIDATE_MSG(hipStreamCreateWithFlags(&c.side.stream, hipStreamNonBlocking) == hipSuccess,
+                "cannot create a stream for an execution context");
+            TRTAMD_VALIDATE(hipEventCreateWithFlags(&c.side.fork, hipEventDisableTiming) == hipSuccess);
+            TRTAMD_VALIDATE(hipEventCreateWithFlags(&c.side.join, hipEventDisableTiming) == hipSuccess);
+            mContexts.push_back(std::move(c));
+        }
+    }
+
+    int32_t contexts() const
+    {
+        return static_cast<int32_t>(mContexts.size());
     }
 
     // emb fp16 | x | qkv | ctx | ao | h | m | f | dummy | emb's second output
@@ -216,11 +273,83 @@ public:
     int enqueue(int32_t const* ids, int32_t const* segs, int32_t const* cu, int32_t batch, int32_t tokens,
         void* workspace, trtamd_half_t* out, hipStream_t stream)
     {
-        TRTAMD_VALIDATE_MSG(mEmbedding != nullptr, "set_embedding has not been called");
+        requireComplete();
+        return enqueueOn(mContexts[0], ids, segs, cu, batch, tokens, workspace, out, stream);
+    }
+
+    // Several independent batches at once: part 0 on the caller's stream, part i on the stream of context i, which
+    // starts behind everything the caller's stream holds so far (fork event) and which the caller's stream waits for
+    // before anything enqueued after this call (join event).  To the caller the whole call is work on `stream`; it
+    // only launches and records, so it can be captured into a graph like the single enqueue.
+    int enqueueConcurrent(trtamd_encoder_batch const* parts, int32_t count, hipStream_t stream)
+    {
+        requireComplete();
+        TRTAMD_VALIDATE_MSG(parts != nullptr && count >= 1 && count <= contexts(),
+            "more parts than reserved execution contexts (trtamd_encoder_reserve_contexts)");
+        for (int32_t i = 1; i < count; ++i)
+        {
+            Side const& sd = mContexts[static_cast<size_t>(i)].side;
+            TRTAMD_VALIDATE(hipEventRecord(sd.fork, stream) == hipSuccess);
+            TRTAMD_VALIDATE(hipStreamWaitEvent(sd.stream, sd.fork, 0) == hipSuccess);
+        }
+        for (int32_t i = 0; i < count; ++i)
+        {
+            trtamd_encoder_batch const& b = parts[i];
+            Context& c = mContexts[static_cast<size_t>(i)];
+            enqueueOn(c, b.ids, b.segment_ids, b.cu_seqlens, b.batch, b.tokens, b.workspace, b.out,
+                i == 0 ? stream : c.side.stream);
+        }
+        for (int32_t i = 1; i < count; ++i)
+        {
+            Side const& sd = mContexts[static_cast<size_t>(i)].side;
+            TRTAMD_VALIDATE(hipEventRecord(sd.join, sd.stream) == hipSuccess);
+            TRTAMD_VALIDATE(hipStreamWaitEvent(stream, sd.join, 0) == hipSuccess);
+        }
+        return TRTAMD_STATUS_SUCCESS;
+    }
+
+    ~Encoder()
+    {
+        for (Context& c : mContexts)
+        {
+            if (c.side.stream)
+            {
+                (void) hipStreamSynchronize(c.side.stream);
+                (void) hipStreamDestroy(c.side.stream);
+                (void) hipEventDestroy(c.side.fork);
+                (void) hipEventDestroy(c.side.join);
+            }
+        }
+    }
+
+private:
+    static constexpr int32_t kMaxContexts = 8;
+
+    struct Side
+    {
+        hipStream_t stream{nullptr};
+        hipEvent_t fork{nullptr}, join{nullptr};
+    };
+
+    struct Context
+    {
+        PluginPtr embedding;
+        std::vector<LayerPlugins> layers;
+        Side side;
+    };
+
+    void requireComplete() const
+    {
+        TRTAMD_VALIDATE_MSG(mContexts[0].embedding != nullptr, "set_embedding has not been called");
         for (Layer const& L : mLayers)
         {
             TRTAMD_VALIDATE_MSG(L.set, "set_layer has not been called for every layer");
         }
+    }
+
+    int enqueueOn(Context& context, int32_t const* ids, int32_t const* segs, int32_t const* cu, int32_t batch,
+        int32_t tokens, void* workspace, trtamd_half_t* out, hipStream_t stream)
+    {
         TRTAMD_VALIDATE(ids && segs && cu && workspace && out && batch > 0 && tokens > 0);
         TRTAMD_VALIDATE_MSG((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "workspace must be 256-byte aligned");
         int64_t const T = tokens, B = batch, E = mCfg.hidden, F = mCfg.ffn;
@@ -257,7 +386,7 @@ public:
         auto const lin = TensorFormat::kLINEAR;
         auto const il = TensorFormat::kCHW32;
 
-        run(mEmbedding,
+        run(context.embedding,
             {desc({T}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f),
                 desc({B + 1}, DataType::kINT32, lin, 1.f), desc({mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
             {desc({T, E, 1, 1}, DataType::kHALF, lin, 1.f), desc({}, DataType::kINT32, lin, 1.f)}, {ids, segs, cu, dummy},
@@ -265,19 +394,21 @@ public:
         checkKernelStatus(trtamd_quantize_fp16_to_interleaved(stream, tokens, mCfg.hidden, emb, mEmbScale, x), "quantise");
 
         float lastScale = mEmbScale;
-        for (Layer const& L : mLayers)
+        for (size_t li = 0; li < mLayers.size(); ++li)
         {
+            Layer const& L = mLayers[li];
+            LayerPlugins const& P = context.layers[li];
             checkKernelStatus(L.qkv.run(stream, x, qkv, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "QKV projection");
-            run(L.attention,
+            run(P.attention,
                 {desc({1, 3 * E, T, 1}, DataType::kINT8, il, L.sQkv), desc({B + 1}, DataType::kINT32, lin, 1.f),
                     desc({mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
                 {desc({1, E, T, 1}, DataType::kINT8, il, L.sCtx)}, {qkv, cu, dummy}, {ctx}, "QKV-to-context");
             checkKernelStatus(L.proj.run(stream, ctx, ao, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "output projection");
-            run(L.ln1, {desc({1, E, T, 1}, DataType::kINT8, il, L.sAo), desc({1, E, T, 1}, DataType::kINT8, il, L.sX)},
+            run(P.ln1, {desc({1, E, T, 1}, DataType::kINT8, il, L.sAo), desc({1, E, T, 1}, DataType::kINT8, il, L.sX)},
                 {desc({1, E, T, 1}, DataType::kINT8, il, L.sH)}, {ao, x}, {h}, "SkipLayerNorm 1");
             checkKernelStatus(L.ffn1.run(stream, h, m, tokens, TRTAMD_LINEAR_GELU, L.ffn1OutScale), "feed-forward 1");
             checkKernelStatus(L.ffn2.run(stream, m, f, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "feed-forward 2");
-            run(L.ln2, {desc({1, E, T, 1}, DataType::kINT8, il, L.sF), desc({1, E, T, 1}, DataType::kINT8, il, L.sH)},
+            run(P.ln2, {desc({1, E, T, 1}, DataType::kINT8, il, L.sF), desc({1, E, T, 1}, DataType::kINT8, il, L.sH)},
                 {desc({1, E, T, 1}, DataType::kINT8, il, L.sOut)}, {f, h}, {x}, "SkipLayerNorm 2");
             lastScale = L.sOut;
         }
@@ -285,11 +416,10 @@ public:
         return TRTAMD_STATUS_SUCCESS;
     }
 
-private:
     trtamd_encoder_config mCfg;
-    PluginPtr mEmbedding;
     float mEmbScale{0.f};
     std::vector<Layer> mLayers;
+    std::vector<Context> mContexts; // [0]: the plugin objects set_embedding / set_layer create
 };
 
 template <typename Fn>
@@ -359,5 +489,23 @@ extern "C" int trtamd_encoder_enqueue(trtamd_encoder_t encoder, int32_t const* i
         TRTAMD_VALIDATE(encoder != nullptr);
         return static_cast<Encoder*>(encoder)->enqueue(ids, segment_ids, cu_seqlens, batch, tokens, workspace, out,
             trtamd::as_stream(stream));
+    });
+}
+
+extern "C" int trtamd_encoder_reserve_contexts(trtamd_encoder_t encoder, int32_t count)
+{
+    return guarded("encoder_reserve_contexts", [&] {
+        TRTAMD_VALIDATE(encoder != nullptr);
+        static_cast<Encoder*>(encoder)->reserveContexts(count);
+        return 0;
+    });
+}
+
+extern "C" int trtamd_encoder_enqueue_concurrent(trtamd_encoder_t encoder, trtamd_encoder_batch const* parts,
+    int32_t count, trtamd_stream_t stream)
+{
+    return guarded("encoder_enqueue_concurrent", [&] {
+        TRTAMD_VALIDATE(encoder != nullptr);
+        return static_cast<Encoder*>(encoder)->enqueueConcurrent(parts, count, trtamd::as_stream(stream));
     });
 }

@@ -199,6 +199,7 @@ class Int8BertEncoder:
         self.buf["ids"] = torch.from_numpy(np.ascontiguousarray(ids, np.int32)).cuda()
         self.buf["segs"] = torch.from_numpy(np.ascontiguousarray(segs, np.int32)).cuda()
         self.buf["cu"] = torch.from_numpy(np.ascontiguousarray(cu, np.int32)).cuda()
+        self._concurrent = None   # its sub-batches point into the tensors replaced above
 
     # ---- single operations -----------------------------------------------------------------------------
     def _check(self, st, what):
@@ -404,6 +405,52 @@ class Int8BertEncoder:
                                       self.stream if stream is None else stream))
         return b["out_native"]
 
+    def prepare_concurrent(self, parts: int = 2):
+        """The caller's side of enqueue_native_concurrent: the bound batch cut into `parts` runs of whole sequences with
+        about the same number of tokens, each with its own cu_seqlens and workspace; execution contexts reserved."""
+        torch, api, b = self.torch, self.api, self.buf
+        if getattr(self, "_native", None) is None:
+            self.build_native()
+        self.prepare_native()
+        cu = b["cu"].cpu().numpy().astype(np.int64)
+        parts = max(1, min(parts, self.B))
+        cuts = [0]
+        for i in range(1, parts):
+            # the sequence boundary nearest to i / parts of the tokens that leaves every part at least one sequence
+            lo, hi = cuts[-1] + 1, self.B - (parts - i)
+            cuts.append(lo + int(np.argmin(np.abs(cu[lo:hi + 1] - cu[-1] * i / parts))))
+        cuts.append(self.B)
+        api.check(api.encoder_reserve_contexts(self._native, max(len(cuts) - 1, 1)))
+        batches = (capi.EncoderBatch * (len(cuts) - 1))()
+        keep = []
+        E = self.cfg.hidden
+        for i in range(len(cuts) - 1):
+            lo, hi = cuts[i], cuts[i + 1]
+            t0, t1 = int(cu[lo]), int(cu[hi])
+            sub_cu = torch.from_numpy((cu[lo:hi + 1] - cu[lo]).astype(np.int32)).cuda()
+            ws = torch.empty((api.encoder_workspace_size(self._native, t1 - t0),), dtype=torch.uint8, device="cuda")
+            keep += [sub_cu, ws]
+            q = batches[i]
+            q.ids = b["ids"].data_ptr() + 4 * t0
+            q.segment_ids = b["segs"].data_ptr() + 4 * t0
+            q.cu_seqlens = sub_cu.data_ptr()
+            q.batch, q.tokens = hi - lo, t1 - t0
+            q.workspace = ws.data_ptr()
+            q.out = b["out_native"].data_ptr() + 2 * E * t0
+        self._concurrent = (batches, len(cuts) - 1, keep)
+        return len(cuts) - 1
+
+    def enqueue_native_concurrent(self, parts: int = 2, stream=None):
+        """One forward pass of the bound batch as `parts` sub-batches that the C++ runner executes at the same time
+        (trtamd_encoder_enqueue_concurrent).  Sequences do not interact, so the output tensor holds the same bits as
+        enqueue_native's; the sub-batches fill the compute units that each other's kernel tails leave idle."""
+        if getattr(self, "_concurrent", None) is None or self._concurrent[1] != parts:
+            self.prepare_concurrent(parts)
+        batches, n, _ = self._concurrent
+        self.api.check(self.api.encoder_enqueue_concurrent(self._native, batches, n,
+                                                           self.stream if stream is None else stream))
+        return self.buf["out_native"]
+
     def prepare_native(self):
         """The caller's side of an enqueue that must not allocate: workspace and output tensor for the bound batch."""
         torch, b = self.torch, self.buf
@@ -418,6 +465,7 @@ class Int8BertEncoder:
         if h:
             self.api.encoder_destroy(h)
             self._native = None
+            self._concurrent = None
 
     def __del__(self):
         h = getattr(self, "_native", None)

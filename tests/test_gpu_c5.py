@@ -196,3 +196,8 @@ def test_native_runner_at_c5_size(c5_layer):
     torch.cuda.synchronize()
     assert np.array_equal(got.cpu().numpy(), out)
     assert np.isfinite(out.astype(np.float32)).all()
+    # the same batch as two halves that run at the same time (the benchmark's default): same bytes
+    got.fill_(float("nan"))
+    got = enc.enqueue_native_concurrent(2)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), out)

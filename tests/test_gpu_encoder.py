@@ -185,3 +185,54 @@ def test_first_enqueue_of_a_fresh_runner_can_be_captured(setup):
         torch.cuda.synchronize()
         assert np.array_equal(result.cpu().numpy(), out), f"replay {k}"
     enc.enqueue(ids, segs, cu)
+
+
+@pytest.mark.parametrize("parts", [2, 3])
+def test_concurrent_sub_batches_give_the_single_pass_bytes(setup, parts):
+    """The batch cut into runs of whole sequences that the runner executes at the same time (one execution context,
+    i.e. one set of plugin clones, per run; side streams forked from and joined to the caller's stream) must give the
+    bytes of the single enqueue, eagerly and on every replay of a captured graph with eager work in between."""
+    import torch
+    cfg, enc, ids, segs, cu, cap, out = setup
+    enc.enqueue_native(ids, segs, cu)
+    torch.cuda.synchronize()
+    n = enc.prepare_concurrent(parts)
+    assert n == parts
+    result = enc.buf["out_native"]
+    for _ in range(2):
+        result.fill_(float("nan"))
+        got = enc.enqueue_native_concurrent(parts)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), out)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            enc.enqueue_native_concurrent(parts, stream=stream.cuda_stream)
+    r = rng(29)
+    ids2 = r.integers(0, cfg.vocab, ids.size).astype(np.int32)
+    d_ids = enc.buf["ids"]
+    d_ids.copy_(torch.from_numpy(ids2))
+    want2 = enc.enqueue_native().cpu().numpy()
+    assert not np.array_equal(want2, out)
+    for k, (tokens, want) in enumerate([(ids, out), (ids2, want2), (ids, out)]):
+        d_ids.copy_(torch.from_numpy(tokens))
+        result.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(result.cpu().numpy(), want), f"replay {k}"
+    enc.enqueue(ids, segs, cu)   # leave the fixture's buffers as the other tests expect them
+
+
+def test_concurrent_enqueue_refuses_more_parts_than_contexts(setup):
+    from tensorrt_amd import capi
+    cfg, enc, ids, segs, cu, cap, out = setup
+    enc.enqueue_native(ids, segs, cu)
+    enc.prepare_concurrent(2)
+    batches, n, _ = enc._concurrent
+    three = (capi.EncoderBatch * 9)()
+    st = enc.api.encoder_enqueue_concurrent(enc._native, three, 9, enc.stream)
+    assert st != 0 and "contexts" in enc.api.last_error_str()
+    assert enc.api.encoder_reserve_contexts(enc._native, 9) != 0
+    enc.enqueue(ids, segs, cu)
