@@ -1,9 +1,9 @@
 """Turns the raw rocprofv3 output of the profile commands into the figures bench.py and profiles/ quote.
 
     python -m tensorrt_amd.profile_summary --workload encoder \\
-        --stats gpurun_out/enc_stats/bench_kernel_stats.csv \\
-        --fetch gpurun_out/enc_fetch/bench_counter_collection.csv \\
-        --write gpurun_out/enc_write/bench_counter_collection.csv [--update profiles/traffic.json]
+        --stats out/enc_stats/bench_kernel_stats.csv \\
+        --fetch out/enc_fetch/bench_counter_collection.csv \\
+        --write out/enc_write/bench_counter_collection.csv [--update profiles/traffic.json]
 
 The FETCH_SIZE / WRITE_SIZE runs must have been made with bench.py's --pmc-calibration, whose plain copy of known
 size (256 MiB read, 256 MiB written) is the yardstick the counter readings are scaled by.  Prints the per-kernel
