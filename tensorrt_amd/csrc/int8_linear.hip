@@ -639,13 +639,14 @@ __device__ __forceinline__ void linear_tile_run(
 //   per row, 64 contiguous bytes of it); in LDS the 16-byte chunk c of row r sits at chunk c ^ (r / 4), which makes
 //   the fragment reads (16 rows x one chunk per 16 lanes) conflict-free; fragment (block, ks) takes chunks 2 ks and
 //   2 ks + 1 of the block's two units.
-template <bool IL, bool IL_OUT, int EPI, typename Origin>
+template <bool IL, bool IL_OUT, int EPI, int KS, typename Origin>
 __device__ __forceinline__ void linear_tile_run_dma(
     LinearArgs const& p, int const count, Origin origin, uint8_t* __restrict__ lds, float* sScale)
 {
+    static_assert(KS == 2 || (KS == 1 && IL), "32-byte stages are built for the interleaved layout only");
     constexpr int WN = 4, MT = 4, NT = 2, NWAVES = 8;
-    constexpr int AF = (kBigTile / 32) * 2;
-    constexpr int BF = (kBigTile / 32) * 2;
+    constexpr int AF = (kBigTile / 32) * KS;   // 1 KB fragments per operand and stage: KS k-halves of 32 bytes per row block
+    constexpr int BF = (kBigTile / 32) * KS;
     constexpr int LA = AF / NWAVES;
     constexpr int LB = BF / NWAVES;
     constexpr int STAGE = (AF + BF) * 1024;
@@ -678,7 +679,7 @@ __device__ __forceinline__ void linear_tile_run_dma(
         laneOff = (uint32_t) rr * (uint32_t) p.K + chunk * 16u;
     }
     auto unit_base = [&](int u, int row0, int R) -> uint32_t {
-        int const rb = u >> 1, sel = u & 1;
+        int const rb = KS == 2 ? u >> 1 : u, sel = KS == 2 ? u & 1 : 0;
         uint32_t const b = IL ? ((uint32_t) sel * (uint32_t) R + (uint32_t) (row0 + rb * 32)) * 32u
                               : (uint32_t) (row0 + rb * 32 + sel * 16) * (uint32_t) p.K;
         return (uint32_t) __builtin_amdgcn_readfirstlane((int) b);
@@ -695,9 +696,9 @@ __device__ __forceinline__ void linear_tile_run_dma(
             ob[q] = unit_base(q * NWAVES + wave, t0, p.T);
         }
     };
-    uint32_t const stepA = IL ? 2u * (uint32_t) p.N * 32u : 64u;
-    uint32_t const stepB = IL ? 2u * (uint32_t) p.T * 32u : 64u;
-    int const nk = p.K / 64; // a multiple of 4
+    uint32_t const stepA = IL ? (uint32_t) KS * (uint32_t) p.N * 32u : 64u;
+    uint32_t const stepB = IL ? (uint32_t) KS * (uint32_t) p.T * 32u : 64u;
+    int const nk = p.K / (32 * KS); // a multiple of 4
 
     uint32_t oaC[LA], obC[LB], oaN[LA], obN[LB];
     // stage kt of the current tile (or stage kt - nk of the next one) into ring slot `slot`
@@ -721,9 +722,9 @@ __device__ __forceinline__ void linear_tile_run_dma(
 
     AccT<EPI> acc[MT][NT];
     // byte offset, inside a 32-row block's 2 KB, of this lane's 16 bytes of fragment ks
-    int readOff[2];
+    int readOff[KS];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+    for (int ks = 0; ks < KS; ++ks)
     {
         if constexpr (IL)
         {
@@ -738,18 +739,18 @@ __device__ __forceinline__ void linear_tile_run_dma(
     auto multiply = [&](int slot) {
         uint8_t const* base = lds + slot * STAGE;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < KS; ++ks)
         {
             i32x4 fa[MT], fb[NT];
 #pragma unroll
             for (int i = 0; i < MT; ++i)
             {
-                fa[i] = *reinterpret_cast<i32x4 const*>(base + (wm * MT + i) * 2048 + readOff[ks]);
+                fa[i] = *reinterpret_cast<i32x4 const*>(base + (wm * MT + i) * (KS * 1024) + readOff[ks]);
             }
 #pragma unroll
             for (int j = 0; j < NT; ++j)
             {
-                fb[j] = *reinterpret_cast<i32x4 const*>(base + AF * 1024 + (wn * NT + j) * 2048 + readOff[ks]);
+                fb[j] = *reinterpret_cast<i32x4 const*>(base + AF * 1024 + (wn * NT + j) * (KS * 1024) + readOff[ks]);
             }
 #pragma unroll
             for (int i = 0; i < MT; ++i)
@@ -949,10 +950,10 @@ __global__ __launch_bounds__(512) void int8_linear_persistent_kernel(LinearArgs 
 }
 
 // The persistent tile plan with direct-to-LDS loads for the 256 x 256 tiles.
-template <bool IL, bool IL_OUT, int EPI>
+template <bool IL, bool IL_OUT, int EPI, int KS = 2>
 __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[4 * 2 * (kBig / 32) * 2 * 1024];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[4 * 2 * (kBig / 32) * KS * 1024];
     __shared__ __attribute__((aligned(16))) float sScale[2 * 2 * kBig];
     if ((int) blockIdx.x < p.persist)
     {
@@ -965,7 +966,7 @@ __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p
             n0 = (int) (pan * pw + rem % pw) * kBig;
             t0 = (int) (rem / pw) * kBig;
         };
-        linear_tile_run_dma<IL, IL_OUT, EPI>(p, count, origin, lds, sScale);
+        linear_tile_run_dma<IL, IL_OUT, EPI, KS>(p, count, origin, lds, sScale);
     }
     else
     {
@@ -1042,6 +1043,19 @@ int launch_shape(hipStream_t stream, LinearArgs a)
         }();
         if constexpr (IL_W == IL_IN && (EPI == kAFFINE || EPI == kGELU || EPI == kF16_AFFINE || EPI == kF16_GELU))
         {
+            static int const stage32 = [] {
+                char const* e = getenv("TRTAMD_LINEAR_STAGE32");
+                return e ? atoi(e) : 0;
+            }();
+            if constexpr (IL_W && (EPI == kAFFINE || EPI == kGELU))
+            {
+                if (stage32 && direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
+                {
+                    hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI, 1>), dim3((uint32_t) pgrid), dim3(512), 0,
+                        stream, a);
+                    return check_launch("int8_linear_dma_kernel(32-byte stages)");
+                }
+            }
             if (direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
             {
                 hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0, stream,
