@@ -292,8 +292,8 @@ int scaled_softmax(hipStream_t stream, int32_t ld, int32_t B, int32_t N, float w
 // addressed by element strides so the same kernel serves Q K^T (B = K read along its rows) and P V.
 // A workgroup of four wavefronts owns a 64 x 64 tile of C, a wavefront a 32 x 32 quarter of it in one accumulator
 // tile of v_mfma_f32_32x32x16_f16 (binary16 operands) or v_mfma_f32_32x32x2_f32 (binary32 operands: full IEEE
-// multiplies).  k advances in chunks of 32 through LDS, both operands stored [row][k] there, so that a fragment
-// is one 16-byte read (binary16) or one 4-byte read per instruction (binary32); rows and k beyond the matrix are
+// multiplies).  k advances in chunks of 64 (binary16) or 32 (binary32) through LDS, both operands stored [row][k]
+// there, so that a fragment is one 16-byte read (binary16) or one 4-byte read per instruction (binary32); rows and k beyond the matrix are
 // zero in LDS, so any M, N, K is served.  Global reads take 16 bytes per lane along whichever dimension is
 // contiguous when addresses and strides allow, single elements otherwise.
 // Batch index z = b*heads + h; operand base = b*batchStride + h*headStride.
@@ -304,23 +304,26 @@ struct GemmOperand
 };
 
 constexpr int kGemmTile = 64; // rows and columns of C per workgroup
-constexpr int kGemmK = 32;    // k per LDS stage
 
 template <typename T>
 struct GemmLds
 {
     // row pitch in elements: 16-byte aligned rows for the binary16 fragment reads, an odd number of dwords for the
     // binary32 ones (consecutive rows then fall in consecutive banks)
-    static constexpr int kPitch = sizeof(T) == 2 ? kGemmK + 8 : kGemmK + 1;
+    // k per LDS stage: the whole head size of 64 in one step for binary16 (one trip to memory and one barrier pair for
+    // Q K^T), 32 for binary32, whose stage of 64 would take the LDS of half the resident workgroups
+    static constexpr int kK = sizeof(T) == 2 ? 64 : 32;
+    static constexpr int kPitch = sizeof(T) == 2 ? kK + 8 : kK + 1;
 };
 
-// One operand's 64 x 32 stage into LDS as [row][k].  rowStride / kStride are the element strides of the operand's
+// One operand's stage (64 rows x one chunk of k) into LDS as [row][k].  rowStride / kStride are the element strides of the operand's
 // row index (m or n) and of k in global memory; rows < rowsLeft and k < kLeft exist.
 template <typename T>
 __device__ inline void stage_operand(T const* __restrict__ g, int64_t const rowStride, int64_t const kStride,
     int const rowsLeft, int const kLeft, bool const vec, T* __restrict__ lds)
 {
     constexpr int P = GemmLds<T>::kPitch;
+    constexpr int kGemmK = GemmLds<T>::kK;
     constexpr int V = 16 / sizeof(T); // elements per 16-byte access
     if (vec && kStride == 1)
     {
@@ -392,6 +395,7 @@ __global__ __launch_bounds__(kBlock) void batched_gemm_kernel(int const M, int c
     GemmOperand const oc, int const vecA, int const vecB)
 {
     constexpr int P = GemmLds<T>::kPitch;
+    constexpr int kGemmK = GemmLds<T>::kK;
     __shared__ __attribute__((aligned(16))) T sA[kGemmTile * P];
     __shared__ __attribute__((aligned(16))) T sB[kGemmTile * P];
     int const z = blockIdx.z;
