@@ -274,7 +274,15 @@ public:
         void* workspace, trtamd_half_t* out, hipStream_t stream)
     {
         requireComplete();
-        return enqueueOn(mContexts[0], ids, segs, cu, batch, tokens, workspace, out, stream);
+        trtamd_encoder_batch const whole{ids, segs, cu, batch, tokens, workspace, out};
+        Pass pass(*this, mContexts[0], whole, stream);
+        pass.embed();
+        for (size_t li = 0; li < mLayers.size(); ++li)
+        {
+            pass.layer(li);
+        }
+        pass.finish();
+        return TRTAMD_STATUS_SUCCESS;
     }
 
     // Several independent batches at once: part 0 on the caller's stream, part i on the stream of context i, which
@@ -286,25 +294,54 @@ public:
         requireComplete();
         TRTAMD_VALIDATE_MSG(parts != nullptr && count >= 1 && count <= contexts(),
             "more parts than reserved execution contexts (trtamd_encoder_reserve_contexts)");
+        std::vector<Pass> passes;
+        passes.reserve(static_cast<size_t>(count));
+        for (int32_t i = 0; i < count; ++i)
+        {
+            Context& c = mContexts[static_cast<size_t>(i)];
+            passes.emplace_back(*this, c, parts[i], i == 0 ? stream : c.side.stream);
+        }
+        // arguments are checked (above) before anything is recorded, so that a refused call leaves no stream forked
         for (int32_t i = 1; i < count; ++i)
         {
             Side const& sd = mContexts[static_cast<size_t>(i)].side;
             TRTAMD_VALIDATE(hipEventRecord(sd.fork, stream) == hipSuccess);
             TRTAMD_VALIDATE(hipStreamWaitEvent(sd.stream, sd.fork, 0) == hipSuccess);
         }
-        for (int32_t i = 0; i < count; ++i)
+        auto join = [&] {
+            bool ok = true;
+            for (int32_t i = 1; i < count; ++i)
+            {
+                Side const& sd = mContexts[static_cast<size_t>(i)].side;
+                ok = hipEventRecord(sd.join, sd.stream) == hipSuccess && ok;
+                ok = hipStreamWaitEvent(stream, sd.join, 0) == hipSuccess && ok;
+            }
+            return ok;
+        };
+        try
         {
-            trtamd_encoder_batch const& b = parts[i];
-            Context& c = mContexts[static_cast<size_t>(i)];
-            enqueueOn(c, b.ids, b.segment_ids, b.cu_seqlens, b.batch, b.tokens, b.workspace, b.out,
-                i == 0 ? stream : c.side.stream);
+            for (Pass& p : passes)
+            {
+                p.embed();
+            }
+            for (size_t li = 0; li < mLayers.size(); ++li)
+            {
+                for (Pass& p : passes)
+                {
+                    p.layer(li);
+                }
+            }
+            for (Pass& p : passes)
+            {
+                p.finish();
+            }
         }
-        for (int32_t i = 1; i < count; ++i)
+        catch (...)
         {
-            Side const& sd = mContexts[static_cast<size_t>(i)].side;
-            TRTAMD_VALIDATE(hipEventRecord(sd.join, sd.stream) == hipSuccess);
-            TRTAMD_VALIDATE(hipStreamWaitEvent(stream, sd.join, 0) == hipSuccess);
+            (void) join(); // a forked stream is joined whatever happened in between
+            throw;
         }
+        TRTAMD_VALIDATE_MSG(join(), "cannot join the execution contexts' streams");
         return TRTAMD_STATUS_SUCCESS;
     }
 
@@ -347,33 +384,54 @@ private:
         }
     }
 
-    int enqueueOn(Context& context, int32_t const* ids, int32_t const* segs, int32_t const* cu, int32_t batch,
-        int32_t tokens, void* workspace, trtamd_half_t* out, hipStream_t stream)
+    // One batch on its way through the network: the buffers carved out of its workspace and the three kinds of step
+    // (embedding, one layer, output).  A single enqueue walks the steps in order; the concurrent one takes the steps of
+    // its parts in turn, layer by layer, so that every stream has work from the first few launches on instead of
+    // part 1 waiting on the host until all of part 0 has been launched.
+    struct Pass
     {
-        TRTAMD_VALIDATE(ids && segs && cu && workspace && out && batch > 0 && tokens > 0);
-        TRTAMD_VALIDATE_MSG((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "workspace must be 256-byte aligned");
-        int64_t const T = tokens, B = batch, E = mCfg.hidden, F = mCfg.ffn;
+        Encoder const& enc;
+        Context& context;
+        hipStream_t stream;
+        int32_t const* ids;
+        int32_t const* segs;
+        int32_t const* cu;
+        int64_t T, B;
+        trtamd_half_t* emb;
+        int8_t *x, *qkv, *ctx, *ao, *h, *m, *f;
+        uint8_t *dummy, *emb2;
+        trtamd_half_t* out;
+        float lastScale;
 
-        auto* base = static_cast<uint8_t*>(workspace);
-        auto carve = [&](size_t bytes) {
-            uint8_t* p = base;
-            base += align256(bytes);
-            return p;
-        };
-        auto* emb = reinterpret_cast<trtamd_half_t*>(carve(T * E * 2));
-        auto* x = reinterpret_cast<int8_t*>(carve(T * E));
-        auto* qkv = reinterpret_cast<int8_t*>(carve(3 * T * E));
-        auto* ctx = reinterpret_cast<int8_t*>(carve(T * E));
-        auto* ao = reinterpret_cast<int8_t*>(carve(T * E));
-        auto* h = reinterpret_cast<int8_t*>(carve(T * E));
-        auto* m = reinterpret_cast<int8_t*>(carve(T * F));
-        auto* f = reinterpret_cast<int8_t*>(carve(T * E));
-        auto* dummy = carve(sizeof(int32_t) * static_cast<size_t>(mCfg.max_seqlen)); // only its extent is read
-        auto* emb2 = carve(256);
+        Pass(Encoder const& e, Context& c, trtamd_encoder_batch const& b, hipStream_t s)
+            : enc(e), context(c), stream(s), ids(b.ids), segs(b.segment_ids), cu(b.cu_seqlens), T(b.tokens), B(b.batch),
+              out(b.out), lastScale(e.mEmbScale)
+        {
+            TRTAMD_VALIDATE(ids && segs && cu && b.workspace && out && b.batch > 0 && b.tokens > 0);
+            TRTAMD_VALIDATE_MSG((reinterpret_cast<uintptr_t>(b.workspace) & 255u) == 0, "workspace must be 256-byte aligned");
+            int64_t const E = enc.mCfg.hidden, F = enc.mCfg.ffn;
+            auto* base = static_cast<uint8_t*>(b.workspace);
+            auto carve = [&](size_t bytes) {
+                uint8_t* p = base;
+                base += align256(bytes);
+                return p;
+            };
+            emb = reinterpret_cast<trtamd_half_t*>(carve(T * E * 2));
+            x = reinterpret_cast<int8_t*>(carve(T * E));
+            qkv = reinterpret_cast<int8_t*>(carve(3 * T * E));
+            ctx = reinterpret_cast<int8_t*>(carve(T * E));
+            ao = reinterpret_cast<int8_t*>(carve(T * E));
+            h = reinterpret_cast<int8_t*>(carve(T * E));
+            m = reinterpret_cast<int8_t*>(carve(T * F));
+            f = reinterpret_cast<int8_t*>(carve(T * E));
+            dummy = carve(sizeof(int32_t) * static_cast<size_t>(enc.mCfg.max_seqlen)); // only its extent is read
+            emb2 = carve(256);
+        }
 
-        auto run = [&](PluginPtr const& plugin, std::vector<PluginTensorDesc> const& in,
-                       std::vector<PluginTensorDesc> const& outDesc, std::vector<void const*> const& inputs,
-                       std::vector<void*> const& outputs, char const* what) {
+        void run(PluginPtr const& plugin, std::vector<PluginTensorDesc> const& in,
+            std::vector<PluginTensorDesc> const& outDesc, std::vector<void const*> const& inputs,
+            std::vector<void*> const& outputs, char const* what) const
+        {
             IPluginV3OneRuntime* rt = runtimeOf(plugin);
             int32_t st = rt->onShapeChange(in.data(), static_cast<int32_t>(in.size()), outDesc.data(),
                 static_cast<int32_t>(outDesc.size()));
@@ -382,26 +440,34 @@ private:
                 st = rt->enqueue(in.data(), outDesc.data(), inputs.data(), outputs.data(), nullptr, stream);
             }
             TRTAMD_VALIDATE_MSG(st == 0, std::string(what) + " failed with status " + std::to_string(st));
-        };
-        auto const lin = TensorFormat::kLINEAR;
-        auto const il = TensorFormat::kCHW32;
+        }
 
-        run(context.embedding,
-            {desc({T}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f),
-                desc({B + 1}, DataType::kINT32, lin, 1.f), desc({mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
-            {desc({T, E, 1, 1}, DataType::kHALF, lin, 1.f), desc({}, DataType::kINT32, lin, 1.f)}, {ids, segs, cu, dummy},
-            {emb, emb2}, "EmbLayerNorm");
-        checkKernelStatus(trtamd_quantize_fp16_to_interleaved(stream, tokens, mCfg.hidden, emb, mEmbScale, x), "quantise");
-
-        float lastScale = mEmbScale;
-        for (size_t li = 0; li < mLayers.size(); ++li)
+        void embed()
         {
-            Layer const& L = mLayers[li];
+            auto const lin = TensorFormat::kLINEAR;
+            int64_t const E = enc.mCfg.hidden;
+            run(context.embedding,
+                {desc({T}, DataType::kINT32, lin, 1.f), desc({T}, DataType::kINT32, lin, 1.f),
+                    desc({B + 1}, DataType::kINT32, lin, 1.f), desc({enc.mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
+                {desc({T, E, 1, 1}, DataType::kHALF, lin, 1.f), desc({}, DataType::kINT32, lin, 1.f)},
+                {ids, segs, cu, dummy}, {emb, emb2}, "EmbLayerNorm");
+            checkKernelStatus(trtamd_quantize_fp16_to_interleaved(stream, static_cast<int32_t>(T), enc.mCfg.hidden, emb,
+                                  enc.mEmbScale, x),
+                "quantise");
+        }
+
+        void layer(size_t li)
+        {
+            auto const lin = TensorFormat::kLINEAR;
+            auto const il = TensorFormat::kCHW32;
+            int64_t const E = enc.mCfg.hidden;
+            int32_t const tokens = static_cast<int32_t>(T);
+            Layer const& L = enc.mLayers[li];
             LayerPlugins const& P = context.layers[li];
             checkKernelStatus(L.qkv.run(stream, x, qkv, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "QKV projection");
             run(P.attention,
                 {desc({1, 3 * E, T, 1}, DataType::kINT8, il, L.sQkv), desc({B + 1}, DataType::kINT32, lin, 1.f),
-                    desc({mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
+                    desc({enc.mCfg.max_seqlen}, DataType::kINT32, lin, 1.f)},
                 {desc({1, E, T, 1}, DataType::kINT8, il, L.sCtx)}, {qkv, cu, dummy}, {ctx}, "QKV-to-context");
             checkKernelStatus(L.proj.run(stream, ctx, ao, tokens, TRTAMD_LINEAR_AFFINE, 1.f), "output projection");
             run(P.ln1, {desc({1, E, T, 1}, DataType::kINT8, il, L.sAo), desc({1, E, T, 1}, DataType::kINT8, il, L.sX)},
@@ -412,9 +478,14 @@ private:
                 {desc({1, E, T, 1}, DataType::kINT8, il, L.sOut)}, {f, h}, {x}, "SkipLayerNorm 2");
             lastScale = L.sOut;
         }
-        checkKernelStatus(trtamd_dequantize_interleaved_to_fp16(stream, tokens, mCfg.hidden, x, lastScale, out), "dequantise");
-        return TRTAMD_STATUS_SUCCESS;
-    }
+
+        void finish()
+        {
+            checkKernelStatus(trtamd_dequantize_interleaved_to_fp16(stream, static_cast<int32_t>(T), enc.mCfg.hidden, x,
+                                  lastScale, out),
+                "dequantise");
+        }
+    };
 
     trtamd_encoder_config mCfg;
     float mEmbScale{0.f};
