@@ -21,8 +21,8 @@ import re
 CALIBRATION_KIB = 256 * 1024
 # bench.py's kernel keys -> a pattern of the kernel's (demangled) name, per workload
 KERNELS = {
-    "encoder": {"ffn1_gemm_gelu": r"int8_linear_dma_kernel<[^>]*,\s*1>", "attention": r"fmha_i8_\w*kernel",
-                "skipln": r"skipln_interleaved_kernel", "gemm_affine": r"int8_linear_dma_kernel<[^>]*,\s*0>"},
+    "encoder": {"ffn1_gemm_gelu": r"int8_linear_dma_kernel<\w+,\s*\w+,\s*1\b", "attention": r"fmha_i8_\w*kernel",
+                "skipln": r"skipln_interleaved_kernel", "gemm_affine": r"int8_linear_dma_kernel<\w+,\s*\w+,\s*0\b"},
     "layer": {"attention": r"fmha_i8_\w*kernel", "skipln": r"skipln_interleaved_kernel"},
 }
 
