@@ -420,12 +420,13 @@ class Int8BertEncoder:
             lo, hi = cuts[-1] + 1, self.B - (parts - i)
             cuts.append(lo + int(np.argmin(np.abs(cu[lo:hi + 1] - cu[-1] * i / parts))))
         cuts.append(self.B)
-        api.check(api.encoder_reserve_contexts(self._native, max(len(cuts) - 1, 1)))
-        batches = (capi.EncoderBatch * (len(cuts) - 1))()
+        # a run of empty sequences has no rows to compute: it is left out
+        runs = [(cuts[i], cuts[i + 1]) for i in range(len(cuts) - 1) if cu[cuts[i + 1]] > cu[cuts[i]]]
+        api.check(api.encoder_reserve_contexts(self._native, max(len(runs), 1)))
+        batches = (capi.EncoderBatch * max(len(runs), 1))()
         keep = []
         E = self.cfg.hidden
-        for i in range(len(cuts) - 1):
-            lo, hi = cuts[i], cuts[i + 1]
+        for i, (lo, hi) in enumerate(runs):
             t0, t1 = int(cu[lo]), int(cu[hi])
             sub_cu = torch.from_numpy((cu[lo:hi + 1] - cu[lo]).astype(np.int32)).cuda()
             ws = torch.empty((api.encoder_workspace_size(self._native, t1 - t0),), dtype=torch.uint8, device="cuda")
@@ -437,16 +438,16 @@ class Int8BertEncoder:
             q.batch, q.tokens = hi - lo, t1 - t0
             q.workspace = ws.data_ptr()
             q.out = b["out_native"].data_ptr() + 2 * E * t0
-        self._concurrent = (batches, len(cuts) - 1, keep)
-        return len(cuts) - 1
+        self._concurrent = (batches, len(runs), keep, parts)
+        return len(runs)
 
     def enqueue_native_concurrent(self, parts: int = 2, stream=None):
         """One forward pass of the bound batch as `parts` sub-batches that the C++ runner executes at the same time
         (trtamd_encoder_enqueue_concurrent).  Sequences do not interact, so the output tensor holds the same bits as
         enqueue_native's; the sub-batches fill the compute units that each other's kernel tails leave idle."""
-        if getattr(self, "_concurrent", None) is None or self._concurrent[1] != parts:
+        if getattr(self, "_concurrent", None) is None or self._concurrent[3] != parts:
             self.prepare_concurrent(parts)
-        batches, n, _ = self._concurrent
+        batches, n = self._concurrent[:2]
         self.api.check(self.api.encoder_enqueue_concurrent(self._native, batches, n,
                                                            self.stream if stream is None else stream))
         return self.buf["out_native"]

@@ -230,9 +230,28 @@ def test_concurrent_enqueue_refuses_more_parts_than_contexts(setup):
     cfg, enc, ids, segs, cu, cap, out = setup
     enc.enqueue_native(ids, segs, cu)
     enc.prepare_concurrent(2)
-    batches, n, _ = enc._concurrent
     three = (capi.EncoderBatch * 9)()
     st = enc.api.encoder_enqueue_concurrent(enc._native, three, 9, enc.stream)
     assert st != 0 and "contexts" in enc.api.last_error_str()
     assert enc.api.encoder_reserve_contexts(enc._native, 9) != 0
+    enc.enqueue(ids, segs, cu)
+
+
+def test_concurrent_enqueue_with_degenerate_batches(setup):
+    """One sequence cannot be cut (one part), and a run of empty sequences has no rows (it is left out): both still
+    give the single enqueue's bytes."""
+    import torch
+    cfg, enc, ids, segs, cu, cap, out = setup
+    r = rng(31)
+    for lens in ([77], [0, 0, 150, 40], [90, 60, 0, 0]):
+        cu2 = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        ids2 = r.integers(0, cfg.vocab, int(cu2[-1])).astype(np.int32)
+        segs2 = r.integers(0, 2, int(cu2[-1])).astype(np.int32)
+        want = enc.enqueue_native(ids2, segs2, cu2).cpu().numpy().copy()
+        n = enc.prepare_concurrent(2)
+        assert n == (1 if len(lens) == 1 else 2)
+        enc.buf["out_native"].fill_(float("nan"))
+        got = enc.enqueue_native_concurrent(2)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), want), lens
     enc.enqueue(ids, segs, cu)
