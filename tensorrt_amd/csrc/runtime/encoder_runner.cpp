@@ -3,6 +3,9 @@
 // stream-ordered sequence of plugin enqueues and linear layers that executes it.  enqueue() only launches, the
 // first call included: every device allocation, copy and kernel attribute happens in set_embedding / set_layer
 // (which run each plugin's first shape change), the activations live in the caller's workspace.
+// Execution contexts (reserve_contexts) are further sets of the plugin objects, cloned, each with a stream and two
+// events; enqueue_concurrent runs one batch per context at the same time, forked from and joined to the caller's
+// stream, and launches the batches' steps in turn so that every stream is fed from the start.
 #include "plugin_common.h"
 #include "trtamd_encoder_runtime.h"
 
