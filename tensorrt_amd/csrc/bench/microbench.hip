@@ -203,6 +203,68 @@ __global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* 
     out[blockIdx.x * kThreads + threadIdx.x] = s + __float_as_int(t);
 }
 
+// The same question across wavefronts: a workgroup of eight wavefronts, two per SIMD (wavefronts w and w + 4 share
+// one), of which the first four issue only MFMAs and the last four only vector-ALU instructions.  `roles` selects who
+// works (1: MFMA wavefronts, 2: vector wavefronts, 3: both); if the two kinds of wavefront ran beside each other,
+// roles 3 would take the longer of the two times, not their sum.
+__global__ __launch_bounds__(512) void mfma_valu_split_kernel(int32_t const* src, int32_t* out, int iters, int nv,
+    int roles)
+{
+    int const wave = threadIdx.x >> 6;
+    int result = 0;
+    if (wave < 4)
+    {
+        if (roles & 1)
+        {
+            i32x4 const a = operand(src, 0), b = operand(src, 1);
+            i32x4 acc[4];
+            for (int i = 0; i < 4; ++i)
+            {
+                acc[i] = i32x4{i, 0, 0, 0};
+            }
+            for (int it = 0; it < iters; ++it)
+            {
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                {
+                    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a), "v"(b));
+                }
+            }
+            for (int i = 0; i < 4; ++i)
+            {
+                result += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+            }
+        }
+    }
+    else if (roles & 2)
+    {
+        float const c = __int_as_float(src[0] & 0x007fffff | 0x3f800000) * 0.5f + 0.25f;
+        float f[8];
+        for (int i = 0; i < 8; ++i)
+        {
+            f[i] = (float) (threadIdx.x & 63) * 0.001f + (float) i;
+        }
+        for (int it = 0; it < iters; ++it)
+        {
+            for (int v = 0; v < nv; v += 8)
+            {
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                {
+                    asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(f[u]) : "v"(c));
+                }
+            }
+        }
+        float t = 0.f;
+        for (int i = 0; i < 8; ++i)
+        {
+            t += f[i];
+        }
+        result = __float_as_int(t);
+    }
+    out[blockIdx.x * 512 + threadIdx.x] = result;
+}
+
 // A kernel that does nothing: what a back-to-back launch of a given grid costs on this box.
 __global__ void empty_kernel(int32_t* out)
 {
@@ -304,4 +366,16 @@ MB_API float trtamd_microbench_valu(int op, int blocks, int iters, int32_t const
     MB_OP(OP_FMA) MB_OP(OP_EXP) MB_OP(OP_ADD) MB_OP(OP_PERM) MB_OP(OP_MAX3) MB_OP(OP_CVT_PK_U8) MB_OP(OP_SOFTMAX_MIX)
 #undef MB_OP
     return -1.f;
+}
+
+// Milliseconds per launch of `blocks` workgroups of eight wavefronts: four that issue 4 * iters MFMAs each and four
+// that issue nv * iters v_fma_f32 each (nv a multiple of 8); roles 1, 2 or 3 as described at the kernel.
+MB_API float trtamd_microbench_mfma_valu_split(int blocks, int iters, int nv, int roles, int32_t const* operands,
+    int32_t* out)
+{
+    return time_launches(
+        [&] {
+            hipLaunchKernelGGL(mfma_valu_split_kernel, dim3(blocks), dim3(512), 0, nullptr, operands, out, iters, nv, roles);
+        },
+        20);
 }

@@ -44,6 +44,8 @@ def _microbench_lib():
     lib.trtamd_microbench_valu.argtypes = [C.c_int] * 3 + [C.c_void_p] * 3
     lib.trtamd_microbench_mfma_valu.restype = C.c_float
     lib.trtamd_microbench_mfma_valu.argtypes = [C.c_int] * 3 + [C.c_void_p] * 2
+    lib.trtamd_microbench_mfma_valu_split.restype = C.c_float
+    lib.trtamd_microbench_mfma_valu_split.argtypes = [C.c_int] * 4 + [C.c_void_p] * 2
     lib.trtamd_microbench_empty.restype = C.c_float
     lib.trtamd_microbench_empty.argtypes = [C.c_int] * 2 + [C.c_void_p]
     return lib
@@ -92,6 +94,13 @@ def microbench(torch, cus: int = 256) -> dict:
         ms = lib.trtamd_microbench_mfma_valu(nv, blocks, iters, rnd.data_ptr(), out.data_ptr())
         co[f"mfma_16x16x64+{nv}_fma"] = round(ms * 1e-3 / (iters * 4 * wps) * clock, 1)
     res["cycles_per_step_mfma_beside_valu"] = co
+    # across wavefronts: per SIMD two wavefronts that only issue MFMAs and two that only issue v_fma_f32 (two workgroups
+    # of eight wavefronts per CU); cycles per iteration (4 MFMAs per MFMA wavefront, 24 fma per vector wavefront)
+    split = {}
+    for roles, name in ((1, "mfma_wavefronts_only"), (2, "vector_wavefronts_only"), (3, "both")):
+        ms = lib.trtamd_microbench_mfma_valu_split(cus * 2, iters, 24, roles, rnd.data_ptr(), out.data_ptr())
+        split[name] = round(ms * 1e-3 / iters * clock, 1)
+    res["cycles_per_iteration_mfma_and_vector_wavefronts_on_one_simd"] = split
     res["empty_launch_us"] = {f"{b}x{t}": round(lib.trtamd_microbench_empty(b, t, out.data_ptr()) * 1e3, 2)
                               for b, t in ((256, 256), (1041, 512), (2048, 256))}
     return res
