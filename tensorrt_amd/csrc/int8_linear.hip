@@ -125,24 +125,50 @@ __device__ __forceinline__ void store_out(void* p, V const& v)
     }
 }
 
+// The 16 scale / offset pairs a lane needs for one 32-channel block (channels 8g + 4 (l/32) + e of the block), read
+// from the tile's vectors in LDS.  For the affine INT8 epilogue the offsets already carry the 128 of the unsigned
+// byte conversion.  A block's scales serve every token block of the same channels, so callers that walk several
+// token blocks load them once.
+struct BlockScales
+{
+    f32x4 al[4], be[4];
+};
+
+template <int EPI>
+__device__ __forceinline__ BlockScales load_block_scales(float const* sAlpha, float const* sBeta)
+{
+    BlockScales s;
+    if constexpr (EPI != kRAW)
+    {
+        int const hi = (threadIdx.x & 63) >> 5;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+        {
+            s.al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + 8 * g + 4 * hi);
+            s.be[g] = *reinterpret_cast<f32x4 const*>(sBeta + 8 * g + 4 * hi);
+            if constexpr (EPI == kAFFINE)
+            {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    s.be[g][e] += 128.f;
+                }
+            }
+        }
+    }
+    return s;
+}
+
 template <bool IL_OUT, int EPI, bool FULL = false, bool THROUGH = false>
-__device__ __forceinline__ void store_block(
-    LinearArgs const& p, AccT<EPI> const& acc, int const c0, int const tb, float const* sAlpha, float const* sBeta)
+__device__ __forceinline__ void store_block_scaled(
+    LinearArgs const& p, AccT<EPI> const& acc, int const c0, int const tb, BlockScales const& sc)
 {
     int const lane = threadIdx.x & 63;
     int const hi = lane >> 5;
     int const t = tb + (lane & 31);
     bool const live = FULL || t < p.T; // FULL: the block lies inside the problem and is stored unconditionally
-    f32x4 al[4], be[4];
-    if constexpr (EPI != kRAW)
-    {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-        {
-            al[g] = *reinterpret_cast<f32x4 const*>(sAlpha + 8 * g + 4 * hi);
-            be[g] = *reinterpret_cast<f32x4 const*>(sBeta + 8 * g + 4 * hi);
-        }
-    }
+    f32x4 const(&al)[4] = sc.al;
+    f32x4 const(&be)[4] = sc.be;
     if constexpr (EPI == kRAW)
     {
         if (live)
@@ -204,7 +230,7 @@ __device__ __forceinline__ void store_block(
                 }
                 else
                 {
-                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf((float) acc[4 * g + e], al[g][e], be[g][e] + 128.f), e, w);
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf((float) acc[4 * g + e], al[g][e], be[g][e]), e, w);
                 }
             }
             d[g] = (int) (w ^ 0x80808080u);
@@ -220,6 +246,13 @@ __device__ __forceinline__ void store_block(
             store_out<THROUGH>(static_cast<int8_t*>(p.out) + o, packed);
         }
     }
+}
+
+template <bool IL_OUT, int EPI, bool FULL = false, bool THROUGH = false>
+__device__ __forceinline__ void store_block(
+    LinearArgs const& p, AccT<EPI> const& acc, int const c0, int const tb, float const* sAlpha, float const* sBeta)
+{
+    store_block_scaled<IL_OUT, EPI, FULL, THROUGH>(p, acc, c0, tb, load_block_scales<EPI>(sAlpha, sBeta));
 }
 
 // Epilogue of one workgroup tile.
@@ -855,6 +888,7 @@ __device__ __forceinline__ void linear_tile_run_dma(
             step(k + 2, S2{}, NoExtra{});
             step(k + 3, S3{}, NoExtra{});
         }
+        BlockScales blockScales;
 #pragma unroll
         for (int i = 0; i < MT; ++i)
         {
@@ -862,8 +896,12 @@ __device__ __forceinline__ void linear_tile_run_dma(
             for (int jj = 0; jj < NT; ++jj)
             {
                 int const cl = (wm * MT + i) * 32;
-                store_block<IL_OUT, EPI, true, IL_OUT && (EPI == kAFFINE || EPI == kGELU)>(p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, scales(j & 1, 0) + cl,
-                    scales(j & 1, 1) + cl);
+                if (jj == 0)
+                {
+                    blockScales = load_block_scales<EPI>(scales(j & 1, 0) + cl, scales(j & 1, 1) + cl);
+                }
+                store_block_scaled<IL_OUT, EPI, true, IL_OUT && (EPI == kAFFINE || EPI == kGELU)>(
+                    p, acc[i][jj], n0 + cl, t0 + (wn * NT + jj) * 32, blockScales);
             }
         }
         n0 = n1;
