@@ -1876,6 +1876,15 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
         int64_t const lds = dataType == 2 ? Lds<1>::total(kt) : Lds<2>::total(kt);
         int64_t const perCu = std::max<int64_t>(1, std::min<int64_t>(dataType == 2 ? 3 : 2, (160 * 1024) / std::max<int64_t>(lds, 1)));
         a.ranked = (int64_t) a.B * a.N * a.qSplit > perCu * 256 ? 1 : 0;
+        // tuning override: TRTAMD_FMHA_RANKED=0 / 1 forces natural order / the longest-first order
+        static int const forcedRank = [] {
+            char const* e = getenv("TRTAMD_FMHA_RANKED");
+            return e ? atoi(e) : -1;
+        }();
+        if (forcedRank >= 0)
+        {
+            a.ranked = forcedRank ? 1 : 0;
+        }
     }
     if (interleaved)
     {
