@@ -127,6 +127,21 @@ class Linear:
         return p
 
 
+def split_runs(cu, parts: int) -> list:
+    """Cuts a packed batch (cu_seqlens `cu`, [B + 1]) into at most `parts` runs of whole sequences with about the same
+    number of tokens each: the i-th cut is the sequence boundary nearest to i / parts of the tokens that still leaves
+    every later run a sequence.  Returns [(first sequence, one past the last)]; runs without tokens are left out."""
+    cu = np.asarray(cu, np.int64)
+    B = len(cu) - 1
+    parts = max(1, min(int(parts), B))
+    cuts = [0]
+    for i in range(1, parts):
+        lo, hi = cuts[-1] + 1, B - (parts - i)
+        cuts.append(lo + int(np.argmin(np.abs(cu[lo:hi + 1] - cu[-1] * i / parts))))
+    cuts.append(B)
+    return [(cuts[i], cuts[i + 1]) for i in range(len(cuts) - 1) if cu[cuts[i + 1]] > cu[cuts[i]]]
+
+
 class Int8BertEncoder:
     """Random-initialised BERT encoder (weights ~N(0, 0.02), LayerNorm gamma ~U(0.5, 1.5), beta ~N(0, 0.1))
     running as INT8 in the 32-interleaved layout."""
@@ -413,15 +428,7 @@ class Int8BertEncoder:
             self.build_native()
         self.prepare_native()
         cu = b["cu"].cpu().numpy().astype(np.int64)
-        parts = max(1, min(parts, self.B))
-        cuts = [0]
-        for i in range(1, parts):
-            # the sequence boundary nearest to i / parts of the tokens that leaves every part at least one sequence
-            lo, hi = cuts[-1] + 1, self.B - (parts - i)
-            cuts.append(lo + int(np.argmin(np.abs(cu[lo:hi + 1] - cu[-1] * i / parts))))
-        cuts.append(self.B)
-        # a run of empty sequences has no rows to compute: it is left out
-        runs = [(cuts[i], cuts[i + 1]) for i in range(len(cuts) - 1) if cu[cuts[i + 1]] > cu[cuts[i]]]
+        runs = split_runs(cu, parts)
         api.check(api.encoder_reserve_contexts(self._native, max(len(runs), 1)))
         batches = (capi.EncoderBatch * max(len(runs), 1))()
         keep = []
