@@ -9,6 +9,8 @@
 #include "host_utils.hpp"
 
 #include <algorithm>
+#include <cmath>
+#include <cstdlib>
 #include <mutex>
 
 // Score matrices of trtamd_unfused_mha_static: device memory that belongs to the library instead of the caller.
@@ -469,10 +471,434 @@ int can_vectorise(T const* base, GemmOperand const& o)
         && o.headStride % V == 0;
 }
 
+// ------------------------------------------------------------------------------------------
+// The same attention in one launch, for sequences whose scores fit in registers (S <= 512, head size <= 128): no
+// score matrix goes to memory.  A workgroup of four wavefronts owns 64 queries of one (batch, head), a wavefront 16
+// of them with ALL their keys, so the row maximum and sum need no exchange between wavefronts.  The matrix products
+// are computed transposed, S^T = K Q^T and O^T = V^T P^T, with the 16 x 16 MFMA tiles: a lane then holds, for its
+// one query, four consecutive keys per tile — the softmax reductions run inside the lane (plus two lane exchanges),
+// and the probabilities are, as they stand in the accumulator registers, the B operand of the second product.  The
+// order in which a lane's eight (binary16) or four (binary32) k positions of a step map to dimensions / keys is
+// free as long as both operands use the same one; it is chosen so that every fragment is one or two whole LDS reads:
+//   binary16  Q K^T step t: lane group g holds dimensions 32t + 8g .. +7;  P V step s of a chunk: keys
+//             32s + 4g .. +3 and 32s + 16 + 4g .. +3 (accumulator tiles 2s and 2s + 1 of the chunk);
+//   binary32  step (u, i): dimension 16u + 4g + i;  P V step (tile j, i): key 16j + 4g + i.
+// K and V pass through one LDS stage of 64 keys, K as [key][dim], V transposed to [dim][key] on the way in (lane =
+// key, so that the transposing writes of a wavefront fall on consecutive addresses).  Numerics as the three-kernel
+// path and the reference's chain of GEMM, softmax, GEMM: scores and probabilities are rounded to T where that chain
+// stores them, accumulation is binary32.  Chunks of 64 keys that lie wholly beyond a batch's valid length are
+// skipped (their probabilities are exactly 0).
+// ------------------------------------------------------------------------------------------
+constexpr int kRegQueries = 64; // queries per workgroup
+constexpr int kRegKeys = 64;    // keys per LDS stage
+constexpr int kRegMaxS = 512;
+constexpr int kRegMaxD = 128;
+
+template <typename T, int DP>
+struct RegLds
+{
+    static constexpr int V = 16 / sizeof(T);
+    // [key][dim]: 16-byte fragment reads of eight consecutive keys fall in different banks
+    static constexpr int kPitchK = sizeof(T) == 2 ? DP + 8 : DP + 4;
+    // [dim][key]: the same for the 8-byte (binary16) and 16-byte (binary32) reads along the keys
+    static constexpr int kPitchV = kRegKeys + 4;
+    static constexpr int kElems = kRegKeys * kPitchK > DP * kPitchV ? kRegKeys * kPitchK : DP * kPitchV;
+};
+
+template <typename T>
+struct RegFrag;
+template <>
+struct RegFrag<f16>
+{
+    typedef f16x8 type;
+};
+template <>
+struct RegFrag<float>
+{
+    typedef f32x4 type;
+};
+
+// V consecutive elements of a row starting at element e0, zero where the row or the element does not exist.
+template <typename T>
+__device__ inline typename RegFrag<T>::type load_piece(T const* __restrict__ row, int const e0, int const n,
+    bool const rowExists, bool const vec)
+{
+    constexpr int V = 16 / sizeof(T);
+    typename RegFrag<T>::type f;
+    if (rowExists && vec && e0 + V <= n)
+    {
+        f = *reinterpret_cast<typename RegFrag<T>::type const*>(row + e0);
+    }
+    else
+    {
+#pragma unroll
+        for (int i = 0; i < V; ++i)
+        {
+            f[i] = (rowExists && e0 + i < n) ? row[e0 + i] : (T) 0.f;
+        }
+    }
+    return f;
+}
+
+// Wavefronts per SIMD the register allocation aims at: what the scores of a query (NT tiles of 4 registers) leave
+// room for without spills.
+template <typename T, int DP, int NT>
+constexpr int reg_waves()
+{
+    constexpr bool wide = sizeof(T) == 4 && DP > 64;
+    return NT <= 8 ? (wide ? 3 : 4) : NT <= 16 ? (wide ? 2 : 3) : 2;
+}
+
+template <typename T, int DP, int NT>
+__global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in_registers_kernel(int const S, int const heads, int const d,
+    int const strips, float const w, T const* __restrict__ qkv, int64_t const ldQKV,
+    int32_t const* __restrict__ maskIdx, T* __restrict__ out, int64_t const ldOut, int const vecIn, int const vecOut)
+{
+    using L = RegLds<T, DP>;
+    using Frag = typename RegFrag<T>::type;
+    constexpr int V = L::V;
+    constexpr int kPieces = DP / V;       // 16-byte pieces of a padded row
+    constexpr int kSteps = DP / (4 * V);  // fragments of a query: 4 lane groups x V dimensions each
+    constexpr int kChunks = NT / 4;       // LDS stages of 64 keys
+    constexpr int kDimTiles = DP / 16;
+    constexpr bool kHalf = sizeof(T) == 2;
+    constexpr int NP = kRegKeys * kPieces / kBlock; // pieces of a stage per thread
+    // stages requested ahead of the one being multiplied, held in registers until their turn in LDS: the binary16
+    // products of a stage are far shorter than a trip to memory, the binary32 ones are not
+    constexpr int D = kHalf ? (DP <= 64 ? 4 : 2) : 1;
+    __shared__ __attribute__((aligned(16))) T lds[L::kElems];
+
+    int const strip = blockIdx.x % strips;
+    int const z = blockIdx.x / strips; // batch * heads + head
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const wave = threadIdx.x >> 6;
+    int const n = lane & 15, g = lane >> 4;
+    int const query = strip * kRegQueries + wave * 16 + n;
+    bool const vec = vecIn != 0;
+    T const* const qp = qkv + (int64_t) z * 3 * d;
+    T const* const kp = qp + d;
+    T const* const vp = qp + 2 * d;
+    int valid = S;
+    if (maskIdx)
+    {
+        valid = max(0, min(S, maskIdx[z / heads]));
+    }
+    int const nChunks = (valid + kRegKeys - 1) / kRegKeys;
+
+    // this lane's part of its query: the B operand of every Q K^T step
+    Frag qf[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t)
+    {
+        qf[t] = load_piece<T>(qp + (int64_t) query * ldQKV, 4 * V * t + V * g, d, query < S, vec);
+    }
+
+    // ---- S^T = K Q^T: tile j of the accumulators holds keys 16 j + 4 g + i of query n ---------------------------
+    Frag ring[D][NP];
+    // K: consecutive threads take the pieces of one key (whole rows per access); V: consecutive threads take
+    // consecutive keys, so that the transposing LDS writes of a wavefront are consecutive
+    auto fetch_k = [&](Frag(&dst)[NP], int const c)
+    {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+        {
+            int const p = threadIdx.x + it * kBlock;
+            int const gk = c * kRegKeys + p / kPieces;
+            dst[it] = load_piece<T>(kp + (int64_t) gk * ldQKV, (p % kPieces) * V, d, gk < S, vec);
+        }
+    };
+    auto fetch_v = [&](Frag(&dst)[NP], int const c)
+    {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+        {
+            int const p = threadIdx.x + it * kBlock;
+            int const gk = c * kRegKeys + p % kRegKeys;
+            dst[it] = load_piece<T>(vp + (int64_t) gk * ldQKV, (p / kRegKeys) * V, d, gk < S, vec);
+        }
+    };
+#pragma unroll
+    for (int c = 0; c < D; ++c)
+    {
+        if (c < nChunks)
+        {
+            fetch_k(ring[c], c);
+        }
+    }
+    f32x4 acc[NT];
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c)
+    {
+        if (c < nChunks)
+        {
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < NP; ++it)
+            {
+                int const p = threadIdx.x + it * kBlock;
+                *reinterpret_cast<Frag*>(&lds[(p / kPieces) * L::kPitchK + (p % kPieces) * V]) = ring[c % D][it];
+            }
+            __syncthreads();
+            if (c + D < kChunks && c + D < nChunks)
+            {
+                fetch_k(ring[c % D], c + D);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < kSteps; ++t)
+                {
+                    if (4 * V * t < d)
+                    {
+                        Frag const kf
+                            = *reinterpret_cast<Frag const*>(&lds[(16 * j + n) * L::kPitchK + 4 * V * t + V * g]);
+                        if constexpr (kHalf)
+                        {
+                            s = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t], s, 0, 0, 0);
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                            {
+                                s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], qf[t][i], s, 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+                acc[4 * c + j] = s;
+            }
+        }
+    }
+
+    // the first V stages are on their way while the softmax runs
+#pragma unroll
+    for (int c = 0; c < D; ++c)
+    {
+        if (c < nChunks)
+        {
+            fetch_v(ring[c], c);
+        }
+    }
+
+    // ---- softmax over the keys of a query: in the lane, then across the four lane groups ------------------------
+    float const wl2 = w * 1.4426950408889634f;
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c)
+    {
+        if (c < nChunks)
+        {
+#pragma unroll
+            for (int j = 4 * c; j < 4 * c + 4; ++j)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    // the score as the GEMM of the three-kernel path stores it
+                    float const x = (float) (T) acc[j][i];
+                    acc[j][i] = 16 * j + 4 * g + i < valid ? x : -3.0e38f;
+                    mx = fmaxf(mx, acc[j][i]);
+                }
+            }
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c)
+    {
+        if (c < nChunks)
+        {
+#pragma unroll
+            for (int j = 4 * c; j < 4 * c + 4; ++j)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    float const e
+                        = 16 * j + 4 * g + i < valid ? __builtin_amdgcn_exp2f((acc[j][i] - mx) * wl2) : 0.f;
+                    acc[j][i] = e;
+                    sum += e;
+                }
+            }
+        }
+    }
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    float const rz = 1.f / sum;
+
+    // ---- O^T = V^T P^T ------------------------------------------------------------------------------------------
+    f32x4 o[kDimTiles];
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt)
+    {
+        o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c)
+    {
+        if (c < nChunks)
+        {
+            // the probabilities of this chunk as the softmax of the three-kernel path stores them
+            T pr[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    pr[j][i] = (T) (16 * (4 * c + j) + 4 * g + i < valid ? acc[4 * c + j][i] * rz : 0.f);
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < NP; ++it)
+            {
+                int const p = threadIdx.x + it * kBlock;
+#pragma unroll
+                for (int i = 0; i < V; ++i)
+                {
+                    lds[((p / kRegKeys) * V + i) * L::kPitchV + p % kRegKeys] = ring[c % D][it][i];
+                }
+            }
+            __syncthreads();
+            if (c + D < kChunks && c + D < nChunks)
+            {
+                fetch_v(ring[c % D], c + D);
+            }
+#pragma unroll
+            for (int dt = 0; dt < kDimTiles; ++dt)
+            {
+                if (16 * dt < d)
+                {
+                    T const* const vrow = &lds[(16 * dt + n) * L::kPitchV];
+                    if constexpr (kHalf)
+                    {
+#pragma unroll
+                        for (int s = 0; s < 2; ++s)
+                        {
+                            f16x4 const lo = *reinterpret_cast<f16x4 const*>(vrow + 32 * s + 4 * g);
+                            f16x4 const hi = *reinterpret_cast<f16x4 const*>(vrow + 32 * s + 16 + 4 * g);
+                            f16x8 const vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                            f16x8 const pf = {pr[2 * s][0], pr[2 * s][1], pr[2 * s][2], pr[2 * s][3],
+                                pr[2 * s + 1][0], pr[2 * s + 1][1], pr[2 * s + 1][2], pr[2 * s + 1][3]};
+                            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                        {
+                            f32x4 const vf = *reinterpret_cast<f32x4 const*>(vrow + 16 * j + 4 * g);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                            {
+                                o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i], pr[j][i], o[dt], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // accumulator i of tile dt: dimension 16 dt + 4 g + i of query n
+    if (query < S)
+    {
+        T* const orow = out + (int64_t) query * ldOut + (int64_t) z * d;
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt)
+        {
+            int const d0 = 16 * dt + 4 * g;
+            T res[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                res[i] = (T) o[dt][i];
+            }
+            if (vecOut && d0 + 4 <= d)
+            {
+                typedef T Tx4 __attribute__((ext_vector_type(4)));
+                *reinterpret_cast<Tx4*>(orow + d0) = Tx4{res[0], res[1], res[2], res[3]};
+            }
+            else
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    if (d0 + i < d)
+                    {
+                        orow[d0 + i] = res[i];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int DP>
+int launch_attention_in_registers(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, T const* qkv,
+    int32_t const* maskIdx, T* output)
+{
+    constexpr int64_t V = 16 / sizeof(T);
+    int64_t const ldQKV = (int64_t) 3 * B * N * d;
+    int64_t const ldOut = (int64_t) B * N * d;
+    int const strips = ceil_div(S, kRegQueries);
+    int64_t const groups = (int64_t) strips * B * N;
+    if (groups > 0x7fffffff)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: %lld workgroups exceed the grid", (long long) groups);
+    }
+    // 16-byte reads of a row's pieces: every row of Q, K and V starts at a multiple of d elements from the base
+    int const vecIn = d % V == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15u) == 0;
+    int const vecOut = d % 4 == 0 && (reinterpret_cast<uintptr_t>(output) & (4 * sizeof(T) - 1)) == 0;
+    float const w = 1.f / sqrtf((float) d);
+    dim3 const grid((unsigned) groups), block(kBlock);
+    int const tiles = ceil_div(S, 16);
+#define TRTAMD_LAUNCH_REG(NT_)                                                                                        \
+    hipLaunchKernelGGL((attention_in_registers_kernel<T, DP, NT_>), grid, block, 0, stream, S, N, d, strips, w, qkv,   \
+        ldQKV, maskIdx, output, ldOut, vecIn, vecOut)
+    if (tiles <= 8)
+    {
+        TRTAMD_LAUNCH_REG(8);
+    }
+    else if (tiles <= 16)
+    {
+        TRTAMD_LAUNCH_REG(16);
+    }
+    else if (tiles <= 24)
+    {
+        TRTAMD_LAUNCH_REG(24);
+    }
+    else
+    {
+        TRTAMD_LAUNCH_REG(32);
+    }
+#undef TRTAMD_LAUNCH_REG
+    return check_launch("attention_in_registers_kernel");
+}
+
+// TRTAMD_UNFUSED_SPLIT=1 keeps every shape on the three kernels with the score matrices in the workspace.
+bool one_launch_allowed()
+{
+    char const* e = getenv("TRTAMD_UNFUSED_SPLIT");
+    return !(e && e[0] == '1');
+}
+
 template <typename T>
 int unfused_mha(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, T const* qkv, int32_t const* maskIdx,
     T* output, void* workspace)
 {
+    if (S <= kRegMaxS && d <= kRegMaxD && one_launch_allowed())
+    {
+        return d <= 64 ? launch_attention_in_registers<T, 64>(stream, S, B, N, d, qkv, maskIdx, output)
+                       : launch_attention_in_registers<T, 128>(stream, S, B, N, d, qkv, maskIdx, output);
+    }
     // geometry of MHARunner::setup (mhaRunner.h:62-83)
     int64_t const ldQKV = (int64_t) 3 * B * N * d;
     int64_t const strideQKV = (int64_t) 3 * d;

@@ -1,4 +1,5 @@
-"""GPU parity of the unfused attention path (scaled/masked softmax, strided batched GEMMs) and of
+"""GPU parity of the unfused attention path (the one-launch kernel that keeps a query's scores in registers for
+S <= 512 and head sizes <= 128, and the strided batched GEMMs around the scaled/masked softmax beyond that) and of
 zeroPadding2d, through the C ABI."""
 import numpy as np
 import pytest
@@ -38,7 +39,10 @@ def test_scaled_softmax(api, dt, S, masked):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
 @pytest.mark.parametrize("S,B,N,d,masked", [(128, 2, 12, 64, True), (20, 3, 2, 32, True), (77, 1, 3, 48, False),
-                                            (384, 1, 2, 64, True), (5, 2, 1, 8, False), (130, 2, 2, 128, True)])
+                                            (384, 1, 2, 64, True), (5, 2, 1, 8, False), (130, 2, 2, 128, True),
+                                            # the last sizes of the one-launch kernel and the first beyond them
+                                            (512, 1, 2, 64, True), (513, 1, 2, 64, True), (60, 2, 2, 129, True),
+                                            (250, 2, 3, 20, True), (1, 3, 2, 64, False), (65, 1, 1, 100, True)])
 def test_unfused_mha(api, dt, S, B, N, d, masked):
     r = rng(210 + S + d)
     qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
@@ -60,6 +64,68 @@ def test_unfused_mha(api, dt, S, B, N, d, masked):
     closed = attention_f64(t[:, 0, 0, 0], t[:L, 0, 0, 1], t[:L, 0, 0, 2], 1 / np.sqrt(d))
     assert_fp_close(got.reshape(S, B, N, d)[:, 0, 0], closed, what="vs float64",
                     **(dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else dict(atol=4e-3, rtol=1e-2)))
+
+
+def _run_unfused(api, dt, S, B, N, d, qkv, lens):
+    type_id = 0 if dt == np.float32 else 1
+    ws = dev_empty((api.unfused_mha_workspace_size(type_id, S, B, N),), np.uint8)
+    out = dev_empty((S, B, N * d), dt, fill=1)
+    d_len = dev(lens) if lens is not None else None
+    api.check(api.unfused_mha(stream(), type_id, S, B, N, d, ptr(dev(qkv)), ptr(d_len), ptr(out), ptr(ws)))
+    sync()
+    return host(out)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("S,B,N,d", [(384, 3, 4, 64), (200, 2, 2, 128), (97, 2, 3, 40), (512, 1, 2, 32)])
+def test_one_launch_against_the_three_kernels(api, monkeypatch, dt, S, B, N, d):
+    """Both routes round scores and probabilities to the storage type at the same places; what is left between them
+    is the order of the binary32 sums."""
+    r = rng(800 + S + d)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
+    lens = r.integers(1, S + 1, B).astype(np.int32)
+    lens[0] = S
+    monkeypatch.setenv("TRTAMD_UNFUSED_SPLIT", "1")
+    split = _run_unfused(api, dt, S, B, N, d, qkv, lens)
+    monkeypatch.setenv("TRTAMD_UNFUSED_SPLIT", "0")
+    one = _run_unfused(api, dt, S, B, N, d, qkv, lens)
+    tol = dict(atol=2e-6, rtol=2e-5) if dt == np.float32 else dict(atol=1e-3, rtol=2e-3)
+    assert_fp_close(one, split, what="one launch vs three kernels", **tol)
+    assert_fp_close(one, oracle.mha_unfused_fixed(qkv, S, B, N, d, lens), what="vs oracle",
+                    **(dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+@pytest.mark.parametrize("S", [70, 600])
+def test_unfused_mha_batch_without_valid_keys(api, dt, S):
+    """A batch whose mask leaves no key gets exact zeros (every probability is 0), its neighbours are untouched by
+    that; a length beyond S means all of S."""
+    B, N, d = 3, 2, 64
+    r = rng(840 + S)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
+    lens = np.array([0, S + 5, S // 2], np.int32)
+    got = _run_unfused(api, dt, S, B, N, d, qkv, lens)
+    assert not got[:, 0].any()
+    ref = oracle.mha_unfused_fixed(qkv, S, B, N, d, np.array([0, S, S // 2], np.int32))
+    assert_fp_close(got, ref, what="vs oracle", **(dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}))
+
+
+def test_unfused_mha_unaligned_operands(api):
+    """Operands that start 2 bytes off a 16-byte boundary take the element-wise loads and stores."""
+    S, B, N, d = 90, 2, 2, 64
+    r = rng(860)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(np.float16)
+    lens = np.array([90, 31], np.int32)
+    raw_in = dev_empty((qkv.size + 8,), np.float16, fill=0)
+    raw_in[1:1 + qkv.size].copy_(dev(qkv).reshape(-1))
+    raw_out = dev_empty((S * B * N * d + 8,), np.float16, fill=0)
+    ws = dev_empty((api.unfused_mha_workspace_size(1, S, B, N),), np.uint8)
+    api.check(api.unfused_mha(stream(), 1, S, B, N, d, ptr(raw_in) + 2, ptr(dev(lens)), ptr(raw_out) + 2, ptr(ws)))
+    sync()
+    got = host(raw_out)
+    assert got[0] == 0 and not got[1 + S * B * N * d:].any()
+    assert_fp_close(got[1:1 + S * B * N * d].reshape(S, B, N * d), oracle.mha_unfused_fixed(qkv, S, B, N, d, lens),
+                    what="vs oracle")
 
 
 def test_unfused_mha_rejects_int8(api):

@@ -1,7 +1,8 @@
 """trtamd_unfused_mha_static: the unfused attention with the library's own score-matrix array instead of a caller
 workspace, for callers that cannot allocate.  Its output must equal trtamd_unfused_mha's bit for bit (same kernels),
 which in turn is held to the floating-point bar against the oracle here; two calls in a row, the second on a
-smaller input, share the array."""
+smaller input, share the array.  Sequences beyond 512 (or head sizes beyond 128) are the ones whose score matrices
+go through the array; shorter ones run in the one-launch kernel, which keeps the scores in registers."""
 import numpy as np
 import pytest
 
@@ -38,9 +39,17 @@ def _both(api, dt, S, B, N, d, seed):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
 def test_two_calls_in_a_row_second_smaller(api, dt):
-    _both(api, dt, 200, 3, 4, 64, seed=301)     # fills 2 * 200*200 * 12 scores of the array
-    _both(api, dt, 77, 2, 3, 32, seed=302)      # a smaller problem over what the first call left behind
-    _both(api, dt, 200, 3, 4, 64, seed=303)     # and a larger one again
+    _both(api, dt, 640, 2, 3, 64, seed=301)     # fills 2 * 640*640 * 6 scores of the array
+    _both(api, dt, 520, 1, 2, 32, seed=302)     # a smaller problem over what the first call left behind
+    _both(api, dt, 640, 2, 3, 64, seed=303)     # and a larger one again
+    _both(api, dt, 100, 2, 2, 136, seed=304)    # a head size beyond the one-launch kernel
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_two_calls_in_a_row_in_registers(api, dt):
+    _both(api, dt, 200, 3, 4, 64, seed=311)     # no score matrix: nothing of the array is touched
+    _both(api, dt, 77, 2, 3, 32, seed=312)
+    _both(api, dt, 200, 3, 4, 64, seed=313)
 
 
 def test_sizes_beyond_the_array_are_refused(api):
