@@ -147,7 +147,9 @@ TRTAMD_API int trtamd_scaled_softmax_fp16(trtamd_stream_t stream, int32_t ld, in
 
 /* UnfusedMHARunner::run  plugin/bertQKVToContextPlugin/mhaRunner.cu:527-601 with the geometry of
  * MHARunner::setup (plugin/bertQKVToContextPlugin/mhaRunner.h:62-83): qkv [S,B,N,3,d], output
- * [S,B,N,d], maskIdx [B] or NULL, workspace of trtamd_unfused_mha_workspace_size bytes.
+ * [S,B,N,d], maskIdx [B] or NULL, workspace of trtamd_unfused_mha_workspace_size bytes (the reference's two S x S
+ * matrices per batch and head; required, and written only for S > 512 or d > 128 — smaller shapes run in one launch
+ * that keeps a query's scores in registers).
  * type: 0 = fp32, 1 = fp16 (nvinfer1::DataType values). */
 TRTAMD_API size_t trtamd_unfused_mha_workspace_size(int32_t type, int32_t S, int32_t B, int32_t N);
 TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
@@ -159,7 +161,8 @@ TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
  * process ends) instead of a caller workspace.  Neither call allocates, frees or synchronises; the first call on a
  * device looks the array's address up.  A problem whose trtamd_unfused_mha_workspace_size exceeds the capacity is
  * refused with TRTAMD_STATUS_NOT_SUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU
- * (different streams) race; calls on one stream, or ordered by events, are safe. */
+ * (different streams) race; calls on one stream, or ordered by events, are safe.  (The array is touched for the
+ * shapes whose scores go through memory, S > 512 or d > 128; the limit applies to every shape.) */
 TRTAMD_API size_t trtamd_unfused_mha_static_capacity(void);
 TRTAMD_API int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N,
     int32_t d, void const* qkv, int32_t const* maskIdx, void* output);

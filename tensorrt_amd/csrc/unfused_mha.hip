@@ -1,5 +1,6 @@
-// Score-materialising attention for the cases the fused kernels do not cover (FP32, any head
-// size, any sequence length), its row softmax, and the head-size padding copy.
+// Attention for the cases the fused kernels do not cover (FP32, any head size, any sequence
+// length) — in one launch with a query's scores in registers where they fit, through score
+// matrices in a workspace otherwise —, the row softmax, and the head-size padding copy.
 //
 // Replaces UnfusedMHARunner::run (plugin/bertQKVToContextPlugin/mhaRunner.cu:527-601: two
 // cuBLAS strided-batched GEMMs around a softmax kernel), computeScaledSoftmax /
