@@ -250,9 +250,10 @@ int scaled_softmax(hipStream_t stream, int32_t ld, int32_t B, int32_t N, float w
         return set_error(TRTAMD_STATUS_BAD_PARAM, "scaledSoftmax: null pointer");
     }
     int64_t const rpb = (int64_t) N * ld;
-    // rows of whole, aligned 16-byte pieces of up to 512 elements: the vectorised kernel
+    // rows of whole, aligned 16-byte pieces, up to 256 of them (2048 binary16 or 1024 binary32 scores, held in
+    // registers between the read and the write): the vectorised kernel
     constexpr int V = 16 / (int) sizeof(T);
-    if (ld % V == 0 && ld <= 512 && (reinterpret_cast<uintptr_t>(in) & 15) == 0
+    if (ld % V == 0 && ld / V <= 256 && (reinterpret_cast<uintptr_t>(in) & 15) == 0
         && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
     {
         int const pieces = ld / V;
@@ -268,9 +269,13 @@ int scaled_softmax(hipStream_t stream, int32_t ld, int32_t B, int32_t N, float w
         {
             launch_softmax_vec<T, 64, 1>(stream, ld, rows, rpb, w, maskIdx, in, out);
         }
-        else
+        else if (pieces <= 128)
         {
             launch_softmax_vec<T, 64, 2>(stream, ld, rows, rpb, w, maskIdx, in, out);
+        }
+        else
+        {
+            launch_softmax_vec<T, 64, 4>(stream, ld, rows, rpb, w, maskIdx, in, out);
         }
         return check_launch("softmax_rows_vec_kernel");
     }

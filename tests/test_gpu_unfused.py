@@ -17,7 +17,8 @@ def api():
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
-@pytest.mark.parametrize("S,masked", [(16, True), (128, True), (384, False), (100, True), (1000, True), (33, False)])
+@pytest.mark.parametrize("S,masked", [(16, True), (128, True), (384, False), (100, True), (1000, True), (33, False),
+                                      (1024, True), (1536, False), (2048, True), (2056, True)])
 def test_scaled_softmax(api, dt, S, masked):
     r = rng(200 + S)
     B, N = 3, 2
