@@ -703,9 +703,10 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                 {
-                    // the score as the GEMM of the three-kernel path stores it
+                    // the score as the GEMM of the three-kernel path stores it; a masked key gets the most
+                    // negative score, whose exponential below is exactly 0
                     float const x = (float) (T) acc[j][i];
-                    acc[j][i] = 16 * j + 4 * g + i < valid ? x : -3.0e38f;
+                    acc[j][i] = (16 * j + 16 <= valid || 16 * j + 4 * g + i < valid) ? x : -3.0e38f;
                     mx = fmaxf(mx, acc[j][i]);
                 }
             }
@@ -725,8 +726,7 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                 {
-                    float const e
-                        = 16 * j + 4 * g + i < valid ? __builtin_amdgcn_exp2f((acc[j][i] - mx) * wl2) : 0.f;
+                    float const e = __builtin_amdgcn_exp2f((acc[j][i] - mx) * wl2);
                     acc[j][i] = e;
                     sum += e;
                 }
@@ -757,7 +757,7 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                 {
-                    pr[j][i] = (T) (16 * (4 * c + j) + 4 * g + i < valid ? acc[4 * c + j][i] * rz : 0.f);
+                    pr[j][i] = (T) (acc[4 * c + j][i] * rz);
                 }
             }
             __syncthreads();
