@@ -27,7 +27,8 @@ def test_scaled_softmax(api, dt, S, masked):
     out = dev_empty((B, N, S, S), dt, fill=1)
     fn = api.scaled_softmax_fp32 if dt == np.float32 else api.scaled_softmax_fp16
     d_len = dev(lens) if masked else None
-    api.check(fn(stream(), S, B, N, 0.125, ptr(d_len), ptr(dev(x)), ptr(out)))
+    d_x = dev(x)    # held until the result is back: a temporary's memory may be handed out again
+    api.check(fn(stream(), S, B, N, 0.125, ptr(d_len), ptr(d_x), ptr(out)))
     sync()
     got = host(out)
     ref = oracle.scaled_softmax(x, 0.125, lens)
@@ -53,7 +54,8 @@ def test_unfused_mha(api, dt, S, B, N, d, masked):
     ws = dev_empty((ws_bytes,), np.uint8)
     out = dev_empty((S, B, N * d), dt, fill=0)
     d_len = dev(lens) if masked else None
-    api.check(api.unfused_mha(stream(), type_id, S, B, N, d, ptr(dev(qkv)), ptr(d_len), ptr(out), ptr(ws)))
+    d_qkv = dev(qkv)
+    api.check(api.unfused_mha(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(out), ptr(ws)))
     sync()
     got = host(out)
     ref = oracle.mha_unfused_fixed(qkv, S, B, N, d, lens)
@@ -72,7 +74,8 @@ def _run_unfused(api, dt, S, B, N, d, qkv, lens):
     ws = dev_empty((api.unfused_mha_workspace_size(type_id, S, B, N),), np.uint8)
     out = dev_empty((S, B, N * d), dt, fill=1)
     d_len = dev(lens) if lens is not None else None
-    api.check(api.unfused_mha(stream(), type_id, S, B, N, d, ptr(dev(qkv)), ptr(d_len), ptr(out), ptr(ws)))
+    d_qkv = dev(qkv)
+    api.check(api.unfused_mha(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(out), ptr(ws)))
     sync()
     return host(out)
 
@@ -121,7 +124,8 @@ def test_unfused_mha_unaligned_operands(api):
     raw_in[1:1 + qkv.size].copy_(dev(qkv).reshape(-1))
     raw_out = dev_empty((S * B * N * d + 8,), np.float16, fill=0)
     ws = dev_empty((api.unfused_mha_workspace_size(1, S, B, N),), np.uint8)
-    api.check(api.unfused_mha(stream(), 1, S, B, N, d, ptr(raw_in) + 2, ptr(dev(lens)), ptr(raw_out) + 2, ptr(ws)))
+    d_len = dev(lens)
+    api.check(api.unfused_mha(stream(), 1, S, B, N, d, ptr(raw_in) + 2, ptr(d_len), ptr(raw_out) + 2, ptr(ws)))
     sync()
     got = host(raw_out)
     assert got[0] == 0 and not got[1 + S * B * N * d:].any()
@@ -140,7 +144,8 @@ def test_zero_padding_2d(api, spitch, dpitch, height):
     r = rng(220 + spitch)
     src = r.integers(0, 256, height * spitch).astype(np.uint8)
     dst = dev_empty((height * dpitch,), np.uint8, fill=0xAB)
-    api.check(api.zero_padding_2d(ptr(dev(src)), spitch, ptr(dst), dpitch, height, stream()))
+    d_src = dev(src)
+    api.check(api.zero_padding_2d(ptr(d_src), spitch, ptr(dst), dpitch, height, stream()))
     sync()
     assert np.array_equal(host(dst), oracle.zero_padding_2d(src, spitch, dpitch, height))
 
@@ -152,7 +157,8 @@ def test_zero_padding_round_trip_at_attention_size(api):
     rows = T * N * 3
     mid = dev_empty((rows * 128,), np.uint8)
     back = dev_empty((rows * 64,), np.uint8)
-    api.check(api.zero_padding_2d(ptr(dev(src)), 64, ptr(mid), 128, rows, stream()))
+    d_src = dev(src)
+    api.check(api.zero_padding_2d(ptr(d_src), 64, ptr(mid), 128, rows, stream()))
     api.check(api.zero_padding_2d(ptr(mid), 128, ptr(back), 64, rows, stream()))
     sync()
     assert np.array_equal(host(back), src)
