@@ -75,6 +75,43 @@ def test_fp16_attention_at_benchmark_size(api, S):
     assert np.array_equal(moved.view(np.uint16), gather_sequences(full, cu, order).view(np.uint16))
 
 
+@pytest.mark.parametrize("dt", [np.float16, np.float32])
+@pytest.mark.parametrize("S", [128, 384])
+def test_unfused_attention_at_benchmark_size(api, dt, S):
+    """The fixed-length [S, B, N, 3, d] layout of the benchmark shape through the unfused path (the route FP32 and
+    head sizes the fused kernels lack take): sampled batches against the oracle on those batches alone and one head
+    against binary64, and the whole output must follow a permutation of the batches bit for bit."""
+    r = rng(3)
+    B, N = 32, 12
+    lens = r.integers(S // 2, S + 1, B).astype(np.int32)
+    qkv = (r.standard_normal((S, B, 3 * N * D)) / 8).astype(dt)
+    type_id = 0 if dt == np.float32 else 1
+    ws = dev_empty((api.unfused_mha_workspace_size(type_id, S, B, N),), np.uint8)
+
+    def run(x, lens_):
+        d_x, d_len = dev(x), dev(lens_)
+        out = dev_empty((S, B, N * D), dt, fill=0)
+        api.check(api.unfused_mha(stream(), type_id, S, B, N, D, ptr(d_x), ptr(d_len), ptr(out), ptr(ws)))
+        sync()
+        return host(out)
+
+    full = run(qkv, lens)
+    assert np.isfinite(full).all()
+    tol = dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}
+    for b in sample_of(lens, r):
+        ref = oracle.mha_unfused_fixed(qkv[:, b:b + 1], S, 1, N, D, lens[b:b + 1])
+        assert_fp_close(full[:, b:b + 1], ref, what=f"batch {b} vs oracle", **tol)
+        x = qkv[:, b].astype(np.float64).reshape(S, N, 3, D)
+        L = int(lens[b])
+        o = attention_f64(x[:, 5, 0], x[:L, 5, 1], x[:L, 5, 2], 0.125)
+        assert_fp_close(full[:, b, 5 * D:6 * D], o, what=f"batch {b}, head 5 vs float64",
+                        **(dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}))
+    order = r.permutation(B)
+    moved = run(np.ascontiguousarray(qkv[:, order]), lens[order])
+    u = np.uint32 if dt == np.float32 else np.uint16
+    assert np.array_equal(moved.view(u), np.ascontiguousarray(full[:, order]).view(u))
+
+
 def int8_layer_inputs(r, B=64, S=384, N=16):
     lens = r.integers(S // 2, S + 1, B)
     cu = cu_of(lens)
