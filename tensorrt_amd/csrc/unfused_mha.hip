@@ -551,8 +551,8 @@ __device__ inline typename RegFrag<T>::type load_piece(T const* __restrict__ row
 template <typename T, int DP, int NT>
 constexpr int reg_waves()
 {
-    constexpr bool wide = sizeof(T) == 4 && DP > 64;
-    return NT <= 8 ? (wide ? 3 : 4) : NT <= 16 ? (wide ? 2 : 3) : 2;
+    constexpr bool big = DP > 64, bigF32 = big && sizeof(T) == 4;
+    return NT <= 8 ? (big ? 3 : 4) : NT <= 16 ? (bigF32 ? 2 : 3) : 2;
 }
 
 template <typename T, int DP, int NT>
@@ -700,20 +700,31 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 #pragma unroll
             for (int j = 4 * c; j < 4 * c + 4; ++j)
             {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
+                // the scores as the GEMM of the three-kernel path stores them
+                f32x4 x = acc[j];
+                if constexpr (kHalf)
                 {
-                    // the score as the GEMM of the three-kernel path stores it; a masked key gets the most
-                    // negative score, whose exponential below is exactly 0
-                    float const x = (float) (T) acc[j][i];
-                    acc[j][i] = (16 * j + 16 <= valid || 16 * j + 4 * g + i < valid) ? x : -3.0e38f;
-                    mx = fmaxf(mx, acc[j][i]);
+                    x = __builtin_convertvector(__builtin_convertvector(x, f16x4), f32x4);
                 }
+                if (16 * j + 16 > valid)
+                {
+                    // the ragged tile (uniform branch): a masked key gets the most negative score, whose
+                    // exponential below is exactly 0
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        x[i] = 16 * j + 4 * g + i < valid ? x[i] : -3.0e38f;
+                    }
+                }
+                acc[j] = x;
+                mx = fmaxf(fmaxf(mx, fmaxf(x[0], x[1])), fmaxf(x[2], x[3]));
             }
         }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
+    // exp((x - max) w) as one fma per score, the way the reference's kernel forms it (x w - max w)
+    float const nmx = -mx * wl2;
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < kChunks; ++c)
@@ -726,7 +737,7 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                 {
-                    float const e = __builtin_amdgcn_exp2f((acc[j][i] - mx) * wl2);
+                    float const e = __builtin_amdgcn_exp2f(fmaf(acc[j][i], wl2, nmx));
                     acc[j][i] = e;
                     sum += e;
                 }
@@ -750,15 +761,12 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
         if (c < nChunks)
         {
             // the probabilities of this chunk as the softmax of the three-kernel path stores them
-            T pr[4][4];
+            typedef T Tx4 __attribute__((ext_vector_type(4)));
+            Tx4 pr[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                {
-                    pr[j][i] = (T) (acc[4 * c + j][i] * rz);
-                }
+                pr[j] = __builtin_convertvector(acc[4 * c + j] * rz, Tx4);
             }
             __syncthreads();
 #pragma unroll
@@ -789,9 +797,8 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
                         {
                             f16x4 const lo = *reinterpret_cast<f16x4 const*>(vrow + 32 * s + 4 * g);
                             f16x4 const hi = *reinterpret_cast<f16x4 const*>(vrow + 32 * s + 16 + 4 * g);
-                            f16x8 const vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                            f16x8 const pf = {pr[2 * s][0], pr[2 * s][1], pr[2 * s][2], pr[2 * s][3],
-                                pr[2 * s + 1][0], pr[2 * s + 1][1], pr[2 * s + 1][2], pr[2 * s + 1][3]};
+                            f16x8 const vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                            f16x8 const pf = __builtin_shufflevector(pr[2 * s], pr[2 * s + 1], 0, 1, 2, 3, 4, 5, 6, 7);
                             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
                         }
                     }
