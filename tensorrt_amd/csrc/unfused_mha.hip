@@ -506,10 +506,17 @@ struct RegLds
     static constexpr int V = 16 / sizeof(T);
     // [key][dim]: 16-byte fragment reads of eight consecutive keys fall in different banks
     static constexpr int kPitchK = sizeof(T) == 2 ? DP + 8 : DP + 4;
-    // [dim][key]: the same for the 8-byte (binary16) and 16-byte (binary32) reads along the keys
-    static constexpr int kPitchV = kRegKeys + 4;
-    static constexpr int kElems = kRegKeys * kPitchK > DP * kPitchV ? kRegKeys * kPitchK : DP * kPitchV;
+    // binary32 V is stored transposed, [dim][key], with a pitch that keeps the 16-byte reads along the keys apart;
+    // binary16 V stays [key][dim] and the fragments come out of transposing reads (ds_read_tr16_b64: the 16 lanes of
+    // a group address 4 keys x 16 dimensions as 8-byte pieces and lane i receives the 4 keys of dimension i), the
+    // pitch of 32 bytes more than a row puts the 4 keys of a group in different banks
+    static constexpr int kPitchV = sizeof(T) == 2 ? DP + 16 : kRegKeys + 4;
+    static constexpr int kElemsV = sizeof(T) == 2 ? kRegKeys * kPitchV : DP * kPitchV;
+    static constexpr int kElems = kRegKeys * kPitchK > kElemsV ? kRegKeys * kPitchK : kElemsV;
 };
+
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 
 template <typename T>
 struct RegFrag;
@@ -601,8 +608,8 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 
     // ---- S^T = K Q^T: tile j of the accumulators holds keys 16 j + 4 g + i of query n ---------------------------
     Frag ring[D][NP];
-    // K: consecutive threads take the pieces of one key (whole rows per access); V: consecutive threads take
-    // consecutive keys, so that the transposing LDS writes of a wavefront are consecutive
+    // K (and binary16 V): consecutive threads take the pieces of one key (whole rows per access); binary32 V:
+    // consecutive threads take consecutive keys, so that the transposing LDS writes of a wavefront are consecutive
     auto fetch_k = [&](Frag(&dst)[NP], int const c)
     {
 #pragma unroll
@@ -619,8 +626,9 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
         for (int it = 0; it < NP; ++it)
         {
             int const p = threadIdx.x + it * kBlock;
-            int const gk = c * kRegKeys + p % kRegKeys;
-            dst[it] = load_piece<T>(vp + (int64_t) gk * ldQKV, (p / kRegKeys) * V, d, gk < S, vec);
+            int const gk = c * kRegKeys + (kHalf ? p / kPieces : p % kRegKeys);
+            dst[it] = load_piece<T>(vp + (int64_t) gk * ldQKV, (kHalf ? p % kPieces : p / kRegKeys) * V, d, gk < S,
+                vec);
         }
     };
 #pragma unroll
@@ -773,10 +781,17 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
             for (int it = 0; it < NP; ++it)
             {
                 int const p = threadIdx.x + it * kBlock;
-#pragma unroll
-                for (int i = 0; i < V; ++i)
+                if constexpr (kHalf)
                 {
-                    lds[((p / kRegKeys) * V + i) * L::kPitchV + p % kRegKeys] = ring[c % D][it][i];
+                    *reinterpret_cast<Frag*>(&lds[(p / kPieces) * L::kPitchV + (p % kPieces) * V]) = ring[c % D][it];
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < V; ++i)
+                    {
+                        lds[((p / kRegKeys) * V + i) * L::kPitchV + p % kRegKeys] = ring[c % D][it][i];
+                    }
                 }
             }
             __syncthreads();
@@ -795,9 +810,14 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
 #pragma unroll
                         for (int s = 0; s < 2; ++s)
                         {
-                            f16x4 const lo = *reinterpret_cast<f16x4 const*>(vrow + 32 * s + 4 * g);
-                            f16x4 const hi = *reinterpret_cast<f16x4 const*>(vrow + 32 * s + 16 + 4 * g);
-                            f16x8 const vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                            // this lane's address: key 32 s + 4 g + n / 4, dimensions 16 dt + 4 (n % 4) .. + 3;
+                            // it receives keys 32 s + 4 g .. + 3 (and those 16 further) of dimension 16 dt + n
+                            T const* const vb = &lds[(32 * s + 4 * g + (n >> 2)) * L::kPitchV + 16 * dt + 4 * (n & 3)];
+                            i16x4 const lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) vb);
+                            i16x4 const hi
+                                = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vb + 16 * L::kPitchV));
+                            f16x8 const vf = __builtin_bit_cast(
+                                f16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
                             f16x8 const pf = __builtin_shufflevector(pr[2 * s], pr[2 * s + 1], 0, 1, 2, 3, 4, 5, 6, 7);
                             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
                         }
