@@ -489,8 +489,9 @@ int can_vectorise(T const* base, GemmOperand const& o)
 //   binary16  Q K^T step t: lane group g holds dimensions 32t + 8g .. +7;  P V step s of a chunk: keys
 //             32s + 4g .. +3 and 32s + 16 + 4g .. +3 (accumulator tiles 2s and 2s + 1 of the chunk);
 //   binary32  step (u, i): dimension 16u + 4g + i;  P V step (tile j, i): key 16j + 4g + i.
-// K and V pass through one LDS stage of 64 keys, K as [key][dim], V transposed to [dim][key] on the way in (lane =
-// key, so that the transposing writes of a wavefront fall on consecutive addresses).  Numerics as the three-kernel
+// K and V pass through one LDS stage of 64 keys, K as [key][dim]; binary32 V transposed to [dim][key] on the way in
+// (lane = key, so that the transposing writes of a wavefront fall on consecutive addresses), binary16 V as
+// [key][dim] with the transposition left to the fragment reads (ds_read_tr16_b64).  Numerics as the three-kernel
 // path and the reference's chain of GEMM, softmax, GEMM: scores and probabilities are rounded to T where that chain
 // stores them, accumulation is binary32.  Chunks of 64 keys that lie wholly beyond a batch's valid length are
 // skipped (their probabilities are exactly 0).
