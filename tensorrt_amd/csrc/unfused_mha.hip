@@ -924,11 +924,17 @@ bool one_launch_allowed()
     return !(e && e[0] == '1');
 }
 
+// Whether a shape runs in the one-launch kernel (and so needs no score matrices).
+bool scores_in_registers(int32_t S, int32_t d)
+{
+    return S <= kRegMaxS && d <= kRegMaxD && one_launch_allowed();
+}
+
 template <typename T>
 int unfused_mha(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, T const* qkv, int32_t const* maskIdx,
     T* output, void* workspace)
 {
-    if (S <= kRegMaxS && d <= kRegMaxD && one_launch_allowed())
+    if (scores_in_registers(S, d))
     {
         return d <= 64 ? launch_attention_in_registers<T, 64>(stream, S, B, N, d, qkv, maskIdx, output)
                        : launch_attention_in_registers<T, 128>(stream, S, B, N, d, qkv, maskIdx, output);
@@ -1065,9 +1071,11 @@ extern "C" int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, i
     {
         return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
     }
-    // 2 * wordSize * S*S * B*N in 128-bit arithmetic free of overflow: each factor is below 2^31
+    // Shapes of the one-launch kernel keep their scores in registers and touch nothing of the array: no limit for
+    // them.  Otherwise 2 * wordSize * S*S * B*N bytes, in double arithmetic free of overflow (each factor is below 2^31).
+    bool const inRegisters = trtamd::scores_in_registers(S, d);
     double const need = 2.0 * (type == 0 ? 4.0 : 2.0) * (double) S * (double) S * (double) B * (double) N;
-    if (need > (double) kStaticScratchBytes)
+    if (!inRegisters && need > (double) kStaticScratchBytes)
     {
         return set_error(TRTAMD_STATUS_NOT_SUPPORTED,
             "unfused MHA (static scratch): S=%d B=%d N=%d needs %.0f bytes of score matrices, the library's array holds "

@@ -52,6 +52,14 @@ def test_two_calls_in_a_row_in_registers(api, dt):
     _both(api, dt, 200, 3, 4, 64, seed=313)
 
 
+def test_shapes_that_stay_in_registers_have_no_limit(api):
+    """S <= 512 with head size <= 128 needs no score matrix: accepted although the reference's workspace for it would be
+    three times the array."""
+    S, B, N, d = 384, 16, 12, 64
+    assert api.unfused_mha_workspace_size(1, S, B, N) > api.unfused_mha_static_capacity()
+    _both(api, np.float16, S, B, N, d, seed=321)
+
+
 def test_sizes_beyond_the_array_are_refused(api):
     cap = api.unfused_mha_static_capacity()
     assert cap == 32 << 20
