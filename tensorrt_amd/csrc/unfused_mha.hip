@@ -580,7 +580,10 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
     // stages requested ahead of the one being multiplied, held in registers until their turn in LDS: the binary16
     // products of a stage are far shorter than a trip to memory, the binary32 ones are not
     constexpr int D = kHalf ? (DP <= 64 ? 4 : 2) : 1;
-    __shared__ __attribute__((aligned(16))) T lds[L::kElems];
+    // binary16: two LDS stages in turn, so that a stage is written while the one before it is still being read and one
+    // barrier per stage is enough; binary32 (long products per stage, three times the LDS) keeps one stage and two
+    constexpr int kStages = kHalf ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) T ldsAll[kStages * L::kElems];
 
     int const strip = blockIdx.x % strips;
     int const z = blockIdx.x / strips; // batch * heads + head
@@ -646,7 +649,11 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
     {
         if (c < nChunks)
         {
-            __syncthreads();
+            T* const lds = ldsAll + (c % kStages) * L::kElems;
+            if constexpr (kStages == 1)
+            {
+                __syncthreads();
+            }
 #pragma unroll
             for (int it = 0; it < NP; ++it)
             {
@@ -777,7 +784,12 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
             {
                 pr[j] = __builtin_convertvector(acc[4 * c + j] * rz, Tx4);
             }
-            __syncthreads();
+            // the stages go on taking turns behind the last one of K
+            T* const lds = ldsAll + ((nChunks + c) % kStages) * L::kElems;
+            if constexpr (kStages == 1)
+            {
+                __syncthreads();
+            }
 #pragma unroll
             for (int it = 0; it < NP; ++it)
             {
