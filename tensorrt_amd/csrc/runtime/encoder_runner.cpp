@@ -348,27 +348,56 @@ public:
         return TRTAMD_STATUS_SUCCESS;
     }
 
-    ~Encoder()
-    {
-        for (Context& c : mContexts)
-        {
-            if (c.side.stream)
-            {
-                (void) hipStreamSynchronize(c.side.stream);
-                (void) hipStreamDestroy(c.side.stream);
-                (void) hipEventDestroy(c.side.fork);
-                (void) hipEventDestroy(c.side.join);
-            }
-        }
-    }
-
 private:
     static constexpr int32_t kMaxContexts = 8;
 
+    // The stream and the two events of a context beyond the first; owns them.
     struct Side
     {
         hipStream_t stream{nullptr};
         hipEvent_t fork{nullptr}, join{nullptr};
+
+        Side() = default;
+        Side(Side const&) = delete;
+        Side& operator=(Side const&) = delete;
+        Side(Side&& o) noexcept : stream(o.stream), fork(o.fork), join(o.join)
+        {
+            o.stream = nullptr;
+            o.fork = o.join = nullptr;
+        }
+        Side& operator=(Side&& o) noexcept
+        {
+            if (this != &o)
+            {
+                release();
+                stream = o.stream, fork = o.fork, join = o.join;
+                o.stream = nullptr;
+                o.fork = o.join = nullptr;
+            }
+            return *this;
+        }
+        ~Side()
+        {
+            release();
+        }
+        void release() noexcept
+        {
+            if (stream)
+            {
+                (void) hipStreamSynchronize(stream);
+                (void) hipStreamDestroy(stream);
+            }
+            if (fork)
+            {
+                (void) hipEventDestroy(fork);
+            }
+            if (join)
+            {
+                (void) hipEventDestroy(join);
+            }
+            stream = nullptr;
+            fork = join = nullptr;
+        }
     };
 
     struct Context
