@@ -896,7 +896,7 @@ int launch_attention_in_registers(hipStream_t stream, int32_t S, int32_t B, int3
     int64_t const ldOut = (int64_t) B * N * d;
     int const strips = ceil_div(S, kRegQueries);
     int64_t const groups = (int64_t) strips * B * N;
-    if (groups > 0x7fffffff)
+    if (groups * kBlock > 0xffffffffll) // a launch holds fewer than 2^32 threads
     {
         return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: %lld workgroups exceed the grid", (long long) groups);
     }
