@@ -63,14 +63,13 @@ __global__ __launch_bounds__(256) void to_interleaved_kernel(
             if constexpr (FROM_HALF)
             {
                 f16 const* src = static_cast<f16 const*>(in) + (size_t) t * C + c;
-                f16x8 const lo = __builtin_nontemporal_load(reinterpret_cast<f16x8 const*>(src));
-                f16x8 const hi = __builtin_nontemporal_load(reinterpret_cast<f16x8 const*>(src) + 1);
+                f16x8 const lo = *reinterpret_cast<f16x8 const*>(src);
+                f16x8 const hi = *(reinterpret_cast<f16x8 const*>(src) + 1);
                 v = quantize16(lo, hi, scale);
             }
             else
             {
-                v = __builtin_nontemporal_load(
-                    reinterpret_cast<i32x4 const*>(static_cast<int8_t const*>(in) + (size_t) t * C + c));
+                v = *reinterpret_cast<i32x4 const*>(static_cast<int8_t const*>(in) + (size_t) t * C + c);
             }
         }
         *reinterpret_cast<i32x4*>(tile + tile_offset(row, col16)) = v;
@@ -87,8 +86,9 @@ __global__ __launch_bounds__(256) void to_interleaved_kernel(
         if (t < T && cs < C)
         {
             i32x4 const v = *reinterpret_cast<i32x4 const*>(tile + slab * kSlabStride + row * 32 + half * 16);
-            __builtin_nontemporal_store(
-                v, reinterpret_cast<i32x4*>(out + ((size_t) (cs >> 5) * T + t) * 32 + half * 16));
+            // 32 tokens x 32 bytes per wavefront, read next by a GEMM or a plugin: through the L2 like the
+            // interleaved outputs of the other kernels
+            store_through_l2(out + ((size_t) (cs >> 5) * T + t) * 32 + half * 16, v);
         }
     }
 }
@@ -111,8 +111,7 @@ __global__ __launch_bounds__(256) void from_interleaved_kernel(
         i32x4 v = {0, 0, 0, 0};
         if (t < T && cs < C)
         {
-            v = __builtin_nontemporal_load(
-                reinterpret_cast<i32x4 const*>(in + ((size_t) (cs >> 5) * T + t) * 32 + half * 16));
+            v = *reinterpret_cast<i32x4 const*>(in + ((size_t) (cs >> 5) * T + t) * 32 + half * 16);
         }
         *reinterpret_cast<i32x4*>(tile + slab * kSlabStride + row * 32 + half * 16) = v;
     }
@@ -139,12 +138,12 @@ __global__ __launch_bounds__(256) void from_interleaved_kernel(
                 hi[e] = (f16) (i8_to_f32((uint32_t) v[2 + (e >> 2)], e & 3) * scale);
             }
             f16* dst = static_cast<f16*>(out) + (size_t) t * C + c;
-            __builtin_nontemporal_store(lo, reinterpret_cast<f16x8*>(dst));
-            __builtin_nontemporal_store(hi, reinterpret_cast<f16x8*>(dst) + 1);
+            *reinterpret_cast<f16x8*>(dst) = lo;
+            *(reinterpret_cast<f16x8*>(dst) + 1) = hi;
         }
         else
         {
-            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(static_cast<int8_t*>(out) + (size_t) t * C + c));
+            *reinterpret_cast<i32x4*>(static_cast<int8_t*>(out) + (size_t) t * C + c) = v;
         }
     }
 }
