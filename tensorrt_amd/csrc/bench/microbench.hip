@@ -161,19 +161,23 @@ __global__ __launch_bounds__(kThreads) void valu_kernel(int32_t const* src, int3
 }
 
 // One MFMA and NV independent vector-ALU instructions per step, in one wavefront's instruction stream: does the
-// matrix pipe run beside the vector ALU (time = max of the two) or in its place (time = sum)?
-template <int NV>
+// matrix pipe run beside the vector ALU (time = max of the two) or in its place (time = sum)?  KIND selects the vector
+// instructions: 0 = v_fma_f32, 1 = v_exp_f32, 2 = the softmax group fma, exp, add, fma (NV counts instructions, so
+// NV / 4 groups).  Sixteen independent chains, so the vector instructions never wait for each other.  WITH_MFMA = false
+// is the control: the same stream without the MFMA.
+template <int NV, int KIND, bool WITH_MFMA>
 __global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* src, int32_t* out, int iters)
 {
     i32x4 const a = operand(src, 0), b = operand(src, 1);
     float const c = __int_as_float(src[0] & 0x007fffff | 0x3f800000) * 0.5f + 0.25f;
     i32x4 acc[4];
-    float f[8];
+    float f[16];
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
     for (int i = 0; i < 4; ++i)
     {
         acc[i] = i32x4{i, 0, 0, 0};
     }
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 16; ++i)
     {
         f[i] = (float) (threadIdx.x & 63) * 0.001f + (float) i;
     }
@@ -182,11 +186,38 @@ __global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* 
 #pragma unroll
         for (int m = 0; m < 4; ++m)
         {
-            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a), "v"(b));
-#pragma unroll
-            for (int v = 0; v < NV; ++v)
+            if (WITH_MFMA)
             {
-                asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(f[(m * NV + v) & 7]) : "v"(c));
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a), "v"(b));
+            }
+            if (KIND == 2)
+            {
+#pragma unroll
+                for (int v = 0; v < NV / 4; ++v)
+                {
+                    int const k = (m * (NV / 4) + v) & 15;
+                    float e;
+                    asm volatile("v_fma_f32 %0, %1, %2, -1.0" : "=v"(e) : "v"(f[k]), "v"(c));
+                    asm volatile("v_exp_f32 %0, %0" : "+v"(e));
+                    asm volatile("v_add_f32 %0, %0, %1" : "+v"(sum[k & 3]) : "v"(e));
+                    asm volatile("v_fma_f32 %0, %1, %2, %2" : "=v"(f[k]) : "v"(e), "v"(c));
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int v = 0; v < NV; ++v)
+                {
+                    int const k = (m * NV + v) & 15;
+                    if (KIND == 0)
+                    {
+                        asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(f[k]) : "v"(c));
+                    }
+                    else
+                    {
+                        asm volatile("v_exp_f32 %0, %0" : "+v"(f[k]));
+                    }
+                }
             }
         }
     }
@@ -195,8 +226,8 @@ __global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* 
     {
         s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
     }
-    float t = 0.f;
-    for (int i = 0; i < 8; ++i)
+    float t = sum[0] + sum[1] + sum[2] + sum[3];
+    for (int i = 0; i < 16; ++i)
     {
         t += f[i];
     }
@@ -204,11 +235,13 @@ __global__ __launch_bounds__(kThreads) void mfma_valu_mix_kernel(int32_t const* 
 }
 
 // The same question across wavefronts: a workgroup of eight wavefronts, two per SIMD (wavefronts w and w + 4 share
-// one), of which the first four issue only MFMAs and the last four only vector-ALU instructions.  `roles` selects who
-// works (1: MFMA wavefronts, 2: vector wavefronts, 3: both); if the two kinds of wavefront ran beside each other,
-// roles 3 would take the longer of the two times, not their sum.
-__global__ __launch_bounds__(512) void mfma_valu_split_kernel(int32_t const* src, int32_t* out, int iters, int nv,
-    int roles)
+// one), of which the first four issue only MFMAs (4 per iteration, independent accumulators) and the last four only
+// v_fma_f32 (NV per iteration on sixteen independent chains, fully unrolled, so that a vector wavefront alone issues
+// at the rate of the ALU and is not waiting for its own results).  `roles` selects who works (1: MFMA wavefronts,
+// 2: vector wavefronts, 3: both); if the two kinds of wavefront run beside each other, roles 3 takes the longer of
+// the two times, not their sum.
+template <int NV, int PAD>
+__global__ __launch_bounds__(512) void mfma_valu_split_kernel(int32_t const* src, int32_t* out, int iters, int roles)
 {
     int const wave = threadIdx.x >> 6;
     int result = 0;
@@ -228,6 +261,13 @@ __global__ __launch_bounds__(512) void mfma_valu_split_kernel(int32_t const* src
                 for (int m = 0; m < 4; ++m)
                 {
                     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a), "v"(b));
+                    // PAD x 8 idle cycles of this wavefront behind every MFMA (scalar no-ops, which do not use the
+                    // vector issue port): its next MFMA then arrives when the matrix pipe is free again
+#pragma unroll
+                    for (int p = 0; p < PAD; ++p)
+                    {
+                        asm volatile("s_nop 7");
+                    }
                 }
             }
             for (int i = 0; i < 4; ++i)
@@ -239,24 +279,21 @@ __global__ __launch_bounds__(512) void mfma_valu_split_kernel(int32_t const* src
     else if (roles & 2)
     {
         float const c = __int_as_float(src[0] & 0x007fffff | 0x3f800000) * 0.5f + 0.25f;
-        float f[8];
-        for (int i = 0; i < 8; ++i)
+        float f[16];
+        for (int i = 0; i < 16; ++i)
         {
             f[i] = (float) (threadIdx.x & 63) * 0.001f + (float) i;
         }
         for (int it = 0; it < iters; ++it)
         {
-            for (int v = 0; v < nv; v += 8)
-            {
 #pragma unroll
-                for (int u = 0; u < 8; ++u)
-                {
-                    asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(f[u]) : "v"(c));
-                }
+            for (int u = 0; u < NV; ++u)
+            {
+                asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(f[u & 15]) : "v"(c));
             }
         }
         float t = 0.f;
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 16; ++i)
         {
             t += f[i];
         }
@@ -333,20 +370,29 @@ MB_API float trtamd_microbench_empty(int blocks, int threads, int32_t* out)
     return time_launches([&] { hipLaunchKernelGGL(empty_kernel, dim3(blocks), dim3(threads), 0, nullptr, out); }, 200);
 }
 
-// Milliseconds per launch; every wavefront issues iters * 4 steps of (one v_mfma_i32_16x16x64_i8, nv v_fma_f32).
-MB_API float trtamd_microbench_mfma_valu(int nv, int blocks, int iters, int32_t const* operands, int32_t* out)
+// Milliseconds per launch; every wavefront issues iters * 4 steps of (one v_mfma_i32_16x16x64_i8, nv vector
+// instructions of `kind`: 0 = v_fma_f32, 1 = v_exp_f32, 2 = the group fma, exp, add, fma (nv a multiple of 4)).
+// with_mfma = 0 leaves the MFMA out (the control for the same vector instructions alone).
+MB_API float trtamd_microbench_mfma_valu(int nv, int kind, int with_mfma, int blocks, int iters, int32_t const* operands,
+    int32_t* out)
 {
-#define MB_NV(V)                                                                                                       \
-    if (nv == V)                                                                                                       \
+#define MB_NV(V, K)                                                                                                    \
+    if (nv == V && kind == K)                                                                                          \
     {                                                                                                                  \
         return time_launches(                                                                                          \
             [&] {                                                                                                      \
-                hipLaunchKernelGGL((mfma_valu_mix_kernel<V>), dim3(blocks), dim3(kThreads), 0, nullptr, operands, out, \
-                    iters);                                                                                            \
+                if (with_mfma)                                                                                         \
+                    hipLaunchKernelGGL((mfma_valu_mix_kernel<V, K, true>), dim3(blocks), dim3(kThreads), 0, nullptr,   \
+                        operands, out, iters);                                                                         \
+                else                                                                                                   \
+                    hipLaunchKernelGGL((mfma_valu_mix_kernel<V, K, false>), dim3(blocks), dim3(kThreads), 0, nullptr,  \
+                        operands, out, iters);                                                                         \
             },                                                                                                         \
             5);                                                                                                        \
     }
-    MB_NV(0) MB_NV(1) MB_NV(2) MB_NV(3) MB_NV(4) MB_NV(6) MB_NV(8) MB_NV(12)
+#define MB_NVS(K) MB_NV(0, K) MB_NV(4, K) MB_NV(8, K) MB_NV(12, K) MB_NV(16, K) MB_NV(24, K) MB_NV(32, K)
+    MB_NVS(0) MB_NVS(1) MB_NVS(2) MB_NV(1, 0) MB_NV(2, 0) MB_NV(3, 0) MB_NV(6, 0) MB_NV(2, 1) MB_NV(6, 1)
+#undef MB_NVS
 #undef MB_NV
     return -1.f;
 }
@@ -369,13 +415,23 @@ MB_API float trtamd_microbench_valu(int op, int blocks, int iters, int32_t const
 }
 
 // Milliseconds per launch of `blocks` workgroups of eight wavefronts: four that issue 4 * iters MFMAs each and four
-// that issue nv * iters v_fma_f32 each (nv a multiple of 8); roles 1, 2 or 3 as described at the kernel.
-MB_API float trtamd_microbench_mfma_valu_split(int blocks, int iters, int nv, int roles, int32_t const* operands,
+// that issue nv * iters v_fma_f32 each (nv 32 or 64); roles 1, 2 or 3 as described at the kernel; pad = number of
+// 8-cycle scalar no-ops behind every MFMA (0 .. 4).
+MB_API float trtamd_microbench_mfma_valu_split(int blocks, int iters, int nv, int pad, int roles, int32_t const* operands,
     int32_t* out)
 {
-    return time_launches(
-        [&] {
-            hipLaunchKernelGGL(mfma_valu_split_kernel, dim3(blocks), dim3(512), 0, nullptr, operands, out, iters, nv, roles);
-        },
-        20);
+#define MB_SPLIT(V, P)                                                                                                 \
+    if (nv == V && pad == P)                                                                                           \
+    {                                                                                                                  \
+        return time_launches(                                                                                          \
+            [&] {                                                                                                      \
+                hipLaunchKernelGGL((mfma_valu_split_kernel<V, P>), dim3(blocks), dim3(512), 0, nullptr, operands, out, \
+                    iters, roles);                                                                                     \
+            },                                                                                                         \
+            20);                                                                                                       \
+    }
+    MB_SPLIT(32, 0) MB_SPLIT(32, 1) MB_SPLIT(32, 2) MB_SPLIT(32, 3) MB_SPLIT(32, 4)
+    MB_SPLIT(64, 0) MB_SPLIT(64, 1) MB_SPLIT(64, 2) MB_SPLIT(64, 3) MB_SPLIT(64, 4)
+#undef MB_SPLIT
+    return -1.f;
 }

@@ -43,9 +43,9 @@ def _microbench_lib():
     lib.trtamd_microbench_valu.restype = C.c_float
     lib.trtamd_microbench_valu.argtypes = [C.c_int] * 3 + [C.c_void_p] * 3
     lib.trtamd_microbench_mfma_valu.restype = C.c_float
-    lib.trtamd_microbench_mfma_valu.argtypes = [C.c_int] * 3 + [C.c_void_p] * 2
+    lib.trtamd_microbench_mfma_valu.argtypes = [C.c_int] * 5 + [C.c_void_p] * 2
     lib.trtamd_microbench_mfma_valu_split.restype = C.c_float
-    lib.trtamd_microbench_mfma_valu_split.argtypes = [C.c_int] * 4 + [C.c_void_p] * 2
+    lib.trtamd_microbench_mfma_valu_split.argtypes = [C.c_int] * 5 + [C.c_void_p] * 2
     lib.trtamd_microbench_empty.restype = C.c_float
     lib.trtamd_microbench_empty.argtypes = [C.c_int] * 2 + [C.c_void_p]
     return lib
@@ -84,23 +84,41 @@ def microbench(torch, cus: int = 256) -> dict:
     clock = float(np.median(mhz)) * 1e6
     res["shader_clock_MHz_under_vector_load"] = round(clock / 1e6)
     res["cycles_per_wave_instruction"] = {k: round(v * clock, 2) for k, v in valu.items()}
+    res["ns_per_wave_instruction"] = {k: round(v * 1e9, 3) for k, v in valu.items()}
     alone = {}
     for op in (0, 1):
         ms = lib.trtamd_microbench_valu(op, cus, iters, rnd.data_ptr(), out.data_ptr(), clocks.data_ptr())
         alone[names[op]] = round(ms * 1e-3 / (iters * 8) * clock, 2)
     res["cycles_per_wave_instruction_one_wave_per_simd"] = alone
+    # one instruction stream: ns per step of one MFMA followed by n independent vector instructions, and of the same
+    # n vector instructions without the MFMA (the control); four wavefronts per SIMD and one
     co = {}
-    for nv in (0, 4, 8, 12):
-        ms = lib.trtamd_microbench_mfma_valu(nv, blocks, iters, rnd.data_ptr(), out.data_ptr())
-        co[f"mfma_16x16x64+{nv}_fma"] = round(ms * 1e-3 / (iters * 4 * wps) * clock, 1)
-    res["cycles_per_step_mfma_beside_valu"] = co
-    # across wavefronts: per SIMD two wavefronts that only issue MFMAs and two that only issue v_fma_f32 (two workgroups
-    # of eight wavefronts per CU); cycles per iteration (4 MFMAs per MFMA wavefront, 24 fma per vector wavefront)
+    for w in (wps, 1):
+        for kind, kname in ((0, "v_fma_f32"), (1, "v_exp_f32"), (2, "fma,exp,add,fma")):
+            row = {}
+            for nv in (0, 4, 8, 12, 16, 24, 32):
+                t = []
+                for with_mfma in (1, 0):
+                    ms = lib.trtamd_microbench_mfma_valu(nv, kind, with_mfma, cus * w, iters // 2, rnd.data_ptr(),
+                                                         out.data_ptr())
+                    t.append(round(ms * 1e-3 / (iters // 2 * 4 * w) * 1e9, 2))
+                row[str(nv)] = t
+            co[f"{kname},waves_per_simd={w}"] = row
+    res["ns_per_step_[mfma_16x16x64_then_n_vector_instructions,n_vector_instructions_alone]_one_stream"] = co
+    # across wavefronts: per SIMD as many wavefronts that only issue MFMAs (4 per iteration) as wavefronts that only
+    # issue v_fma_f32 (nv per iteration, 16 independent chains); workgroups of eight wavefronts, wgs_per_cu of them
+    # on a CU; ns per iteration and SIMD for the MFMA wavefronts alone, the vector wavefronts alone, and both
     split = {}
-    for roles, name in ((1, "mfma_wavefronts_only"), (2, "vector_wavefronts_only"), (3, "both")):
-        ms = lib.trtamd_microbench_mfma_valu_split(cus * 2, iters, 24, roles, rnd.data_ptr(), out.data_ptr())
-        split[name] = round(ms * 1e-3 / iters * clock, 1)
-    res["cycles_per_iteration_mfma_and_vector_wavefronts_on_one_simd"] = split
+    for wgs in (1, 2):
+        for nv in (32, 64):
+            for pad in (0, 1, 2, 3, 4):
+                t = []
+                for roles in (1, 2, 3):
+                    ms = lib.trtamd_microbench_mfma_valu_split(cus * wgs, iters, nv, pad, roles, rnd.data_ptr(),
+                                                               out.data_ptr())
+                    t.append(round(ms * 1e-3 / iters * 1e9, 1))
+                split[f"wgs_per_cu={wgs},nv={nv},idle_cycles_behind_each_mfma={8 * pad}"] = t
+    res["ns_per_iteration_[mfma_wavefronts_only,vector_wavefronts_only,both]_on_one_simd"] = split
     res["empty_launch_us"] = {f"{b}x{t}": round(lib.trtamd_microbench_empty(b, t, out.data_ptr()) * 1e3, 2)
                               for b, t in ((256, 256), (1041, 512), (2048, 256))}
     return res
