@@ -18,6 +18,7 @@ INCLUDE = os.path.join(os.path.dirname(ROOT), "include")
 LIB_DIR = os.path.join(ROOT, "lib")
 LIB_NAME = "libtrtamd_bert_plugins.so"
 MICROBENCH_LIB_NAME = "libtrtamd_microbench.so"   # instruction-rate probes for bench.py; not part of the plugin library
+ABLATION_LIB_NAME = "libtrtamd_ablation.so"       # the plugin library with the attention MFMAs left out (timing only)
 OBJ_DIR = os.path.join(CSRC, "_obj")
 
 ARCH = "gfx950"
@@ -45,9 +46,9 @@ def sources() -> list[str]:
     return out
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.relpath(src, CSRC).replace(os.sep, "_") + ".o")
-    cmd = [_hipcc(), *COMMON_FLAGS, "-x", "hip", "-c", src, "-o", obj]
+def _compile(src: str, extra: tuple = (), suffix: str = "") -> str:
+    obj = os.path.join(OBJ_DIR, os.path.relpath(src, CSRC).replace(os.sep, "_") + suffix + ".o")
+    cmd = [_hipcc(), *COMMON_FLAGS, *extra, "-x", "hip", "-c", src, "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the AMDGPU feature name and says so; that line is noise
     err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -94,6 +95,34 @@ def build_microbench(verbose: bool = False) -> str:
     return out
 
 
+def build_ablation(verbose: bool = False) -> str:
+    """A diagnostic copy of the plugin library whose cu_seqlens attention kernels leave their MFMAs out
+    (csrc/fused_mha.hip built with -DTRTAMD_ABLATE_ATTENTION_MFMA, every other object as in the plugin library, which
+    must have been built): wrong results, and the time the kernels would take if the matrix work were free.
+    `python -m tensorrt_amd.kernel_bench --ablation` times it; nothing else loads it."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    fused = os.path.join(CSRC, "fused_mha.hip")
+    ablated = _compile(fused, ("-DTRTAMD_ABLATE_ATTENTION_MFMA",), ".ablated")
+    plain = os.path.join(OBJ_DIR, os.path.relpath(fused, CSRC).replace(os.sep, "_") + ".o")
+    objs = []
+    for src in sources():
+        obj = os.path.join(OBJ_DIR, os.path.relpath(src, CSRC).replace(os.sep, "_") + ".o")
+        if not os.path.exists(obj):
+            raise RuntimeError(f"{obj} is missing: build the plugin library first")
+        objs.append(ablated if obj == plain else obj)
+    out = os.path.join(LIB_DIR, ABLATION_LIB_NAME)
+    cmd = [_hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out + ".tmp", *objs, "-ldl", "-lpthread"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    os.replace(out + ".tmp", out)
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build_library(verbose=True)
     build_microbench(verbose=True)
+    if "--ablation" in sys.argv[1:]:
+        build_ablation(verbose=True)

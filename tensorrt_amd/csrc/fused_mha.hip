@@ -55,6 +55,33 @@ __device__ inline float mul_rounded(float a, float b)
     return a * b;
 }
 
+// The MFMAs of the cu_seqlens kernels (fmha_i8_prefix_kernel, fmha_f16_prefix_kernel) go through these wrappers.  A
+// library built with -DTRTAMD_ABLATE_ATTENTION_MFMA (`python -m tensorrt_amd.build --ablation` writes it to
+// lib/libtrtamd_ablation.so; `python -m tensorrt_amd.kernel_bench --ablation` times it; nothing else loads it) leaves
+// the instruction out: the result registers keep what they held and every other instruction of the kernel stays, so
+// the results are wrong and the launch takes what the kernel would take if its matrix work cost nothing.
+__device__ __forceinline__ i32x4 attention_mfma_i8(i32x4 const a, i32x4 const b, i32x4 c)
+{
+#ifdef TRTAMD_ABLATE_ATTENTION_MFMA
+    i32x4 d;
+    asm volatile("; v_mfma_i32_16x16x64_i8 left out" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+#else
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+#endif
+}
+
+__device__ __forceinline__ f32x4 attention_mfma_f16(f16x8 const a, f16x8 const b, f32x4 c)
+{
+#ifdef TRTAMD_ABLATE_ATTENTION_MFMA
+    f32x4 d;
+    asm volatile("; v_mfma_f32_16x16x32_f16 left out" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+#else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
 // x[dt] of the lane in 16-lane row g  ->  x[g'] = what row g' held in its x[g]: a 4 x 4 transpose over the four rows of
 // a wavefront.  All 64 lanes must be active.  The attention kernels end with lane (g, query) holding a piece of each
 // quarter dt of the query's output row; transposed, it holds the whole quarter dt = g and stores it in one piece.
@@ -818,7 +845,7 @@ __device__ __forceinline__ void tile_i8(FmhaArgs const& a, SeqInfo const& sq, in
                 seed[j] = (16 * (t & 3) + j) < lastRel ? kMagicBits : kNegInfBits;
             }
         }
-        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(kreg, qreg, seed, 0, 0, 0);
+        acc[t] = attention_mfma_i8(kreg, qreg, seed);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -938,7 +965,7 @@ __device__ __forceinline__ void tile_i8(FmhaArgs const& a, SeqInfo const& sq, in
             i32x2 const v0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + sc));
             i32x2 const v1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*) (vbase + 32 * kRow + sc));
             i32x4 const vreg = {v0[0], v0[1], v1[0], v1[1]};
-            oacc[dt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(vreg, preg, oacc[dt], 0, 0, 0);
+            oacc[dt] = attention_mfma_i8(vreg, preg, oacc[dt]);
         }
     }
 
@@ -1417,7 +1444,7 @@ __device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq,
             for (int h = 0; h < 2; ++h)
             {
                 f16x8 const kreg = *reinterpret_cast<f16x8 const*>(sK + key * kRow + swz<2>(key, h * 4 + g) * 16);
-                sd = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg, qreg[h], sd, 0, 0, 0);
+                sd = attention_mfma_f16(kreg, qreg[h], sd);
             }
             acc[t] = sd;
         }
@@ -1499,10 +1526,9 @@ __device__ __forceinline__ void attend_f16(FmhaArgs const& a, SeqInfo const& sq,
                     i16x4 const v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vbase + 16 * kRow + sc));
                     typedef short i16x8 __attribute__((ext_vector_type(8)));
                     i16x8 const both = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        __builtin_bit_cast(f16x8, both), preg, oacc[dt], 0, 0, 0);
+                    oacc[dt] = attention_mfma_f16(__builtin_bit_cast(f16x8, both), preg, oacc[dt]);
                 }
-                sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, preg, sacc, 0, 0, 0);
+                sacc = attention_mfma_f16(ones, preg, sacc);
             }
         }
 

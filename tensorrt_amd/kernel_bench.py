@@ -490,14 +490,97 @@ def extra_rows(api, torch, steps: int = 100) -> list:
     return rows
 
 
+def attention_rows(api, torch, steps: int = 200) -> list:
+    """The cu_seqlens attention kernels alone, on device-generated operands: INT8 (interleaved layout) at the encoder's
+    and the layer workload's shapes and with full-length sequences, FP16 at the BERT-base shapes.  Used to time a plugin
+    library against its MFMA-less diagnostic build (`--ablation`), whose results are wrong on purpose."""
+    from tensorrt_amd import capi
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+
+    def timeit(fn):
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.25:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e-3 / steps)
+        return best
+
+    def run(name, lens, N, S, int8):
+        lens = np.asarray(lens)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        T, E = int(cu[-1]), N * 64
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(1)
+        x = torch.randn((T, 3 * E), device="cuda", generator=gen)
+        p = capi.FmhaParams()
+        dcu = torch.from_numpy(cu).cuda()
+        if int8:
+            qkv = torch.clamp(torch.round(x * (127 / 4.5)), -127, 127).to(torch.int8)
+            out = torch.zeros(T * E, dtype=torch.int8, device="cuda")
+            sq = 4.5 / 127
+            p.qkv_stride_in_bytes = p.o_stride_in_bytes = T
+            p.scale_bmm1, p.scale_softmax, p.scale_bmm2 = f32_bits(sq * sq * 0.125), f32_bits(127.0), f32_bits(sq / 127 / 0.01)
+            p.interleaved = 1
+        else:
+            qkv = (x / 8).half()
+            out = torch.zeros((T, E), dtype=torch.float16, device="cuda")
+            p.qkv_stride_in_bytes, p.o_stride_in_bytes = 2 * 3 * E, 2 * E
+            p.scale_bmm1, p.scale_softmax, p.scale_bmm2 = half2_bits(0.125), half2_bits(1.0), half2_bits(1.0)
+        p.qkv_ptr, p.o_ptr, p.cu_seqlens = qkv.data_ptr(), out.data_ptr(), dcu.data_ptr()
+        p.b, p.h, p.s, p.d = len(lens), N, S, 64
+        t = timeit(lambda: api.check(api.fused_mha_run(stream, 2 if int8 else 1, C.byref(p))))
+        ops = 4.0 * 64 * N * float(np.sum(lens.astype(np.float64) ** 2))
+        rows.append({"kernel": name, "gpu_us": round(t * 1e6, 2), "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s",
+                     "frac": round(ops / t / (PEAK_I8 if int8 else PEAK_F16), 4)})
+
+    r = np.random.default_rng(1)
+    run("INT8 v6, 128 sequences U[128,384], 16 heads (encoder)", r.integers(128, 385, 128), 16, 384, True)
+    run("INT8 v6, 64 sequences U[192,384], 16 heads (layer)", np.random.default_rng(1).integers(192, 385, 64), 16, 384, True)
+    run("INT8 v6, 128 sequences of 384, 16 heads", np.full(128, 384), 16, 384, True)
+    run("FP16 v5, 32 sequences U[192,384], 12 heads", np.random.default_rng(1).integers(192, 385, 32), 12, 384, False)
+    run("FP16 v5, 32 sequences U[64,128], 12 heads", np.random.default_rng(1).integers(64, 129, 32), 12, 128, False)
+    run("FP16 v5, 64 sequences of 384, 12 heads", np.full(64, 384), 12, 384, False)
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--ablation", action="store_true",
+                    help="time the cu_seqlens attention kernels of lib/libtrtamd_ablation.so (the MFMAs left out; "
+                         "`python -m tensorrt_amd.build --ablation`) and, in a second process, of the plugin library")
+    ap.add_argument("--attention-only", action="store_true", help="only the attention rows of --ablation, this library")
     args = ap.parse_args()
 
+    if args.ablation:
+        # two libraries that export the same symbols do not go into one process: a child per library
+        import subprocess
+        import sys
+        import tensorrt_amd
+        for lib in (os.path.join(os.path.dirname(tensorrt_amd.library_path()), "libtrtamd_ablation.so"),
+                    tensorrt_amd.library_path()):
+            print(f"== {os.path.basename(lib)}", flush=True)
+            env = dict(os.environ, TRTAMD_KERNEL_BENCH_LIBRARY=lib)
+            subprocess.run([sys.executable, "-m", "tensorrt_amd.kernel_bench", "--attention-only", "--steps",
+                            str(args.steps)], env=env, check=True)
+        return
+
     import torch
+    if os.environ.get("TRTAMD_KERNEL_BENCH_LIBRARY"):
+        import tensorrt_amd
+        tensorrt_amd._LIB = os.environ["TRTAMD_KERNEL_BENCH_LIBRARY"]   # the diagnostic build, this process only
     from tensorrt_amd import capi
     api = capi.api()
     # the GPU raises its clocks over the first tens of milliseconds of load
@@ -507,6 +590,11 @@ def main():
         torch.mm(warm, warm)
         torch.cuda.synchronize()
     del warm
+    if args.attention_only:
+        for row in attention_rows(api, torch, args.steps):
+            print(f"{row['kernel']:60s} {row['gpu_us']:9.2f} us {row['achieved']:9.1f} {row['unit']:>5s} {row['frac']:8.4f}",
+                  flush=True)
+        return
     print(f"{'config':22s} {'kernel':62s} {'shape':44s} {'us':>9s} {'achieved':>14s} {'of peak':>8s} {'CPU ms':>9s}")
     mb = microbench(torch)
     for row in config_rows(api, torch, args.steps, args.seed, cpu=not args.no_cpu,
