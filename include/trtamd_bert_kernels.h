@@ -158,13 +158,16 @@ TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
 /* trtamd_unfused_mha for callers that cannot allocate (code under graph capture, tight serving loops, harnesses
  * that forbid hipMalloc).  No counterpart in the reference: the score matrices live in a device array that belongs to
  * the library (trtamd_unfused_mha_static_capacity() bytes, 32 MiB, held by every GPU the library runs on until the
- * process ends) instead of a caller workspace.  Neither call allocates, frees or synchronises; the first call on a
- * device looks the array's address up.  A problem whose trtamd_unfused_mha_workspace_size exceeds the capacity is
+ * process ends) instead of a caller workspace.  None of the calls allocates, frees or synchronises; the array's address
+ * is looked up once per device, by trtamd_unfused_mha_static_prepare() (call it with that device current before a
+ * stream of that device is put into capture: the look-up may load the library's code object) or else by the first
+ * trtamd_unfused_mha_static on the device.  A problem whose trtamd_unfused_mha_workspace_size exceeds the capacity is
  * refused with TRTAMD_STATUS_NOT_SUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU
  * (different streams) race; calls on one stream, or ordered by events, are safe.  The array is used, and the limit
  * applies, for the shapes whose scores go through memory (S > 512 or d > 128); smaller shapes keep their scores in
  * registers, touch nothing of the array and are accepted at any batch size. */
 TRTAMD_API size_t trtamd_unfused_mha_static_capacity(void);
+TRTAMD_API int trtamd_unfused_mha_static_prepare(void);
 TRTAMD_API int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N,
     int32_t d, void const* qkv, int32_t const* maskIdx, void* output);
 

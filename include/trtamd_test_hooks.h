@@ -24,6 +24,14 @@ extern "C"
 TRTAMD_API int trtamd_fused_mha_run_debug(trtamd_stream_t stream, int32_t data_type, trtamd_fmha_params const* params,
     int32_t* acc1, int8_t* p8);
 
+/* Tuning switches (README, "Tuning switches"): kernel variants other than the default choice.  A process normally
+ * selects them with an environment variable of the same name, read once; these two calls let one test process walk
+ * through the settings instead.  name: the variable's name, e.g. "TRTAMD_LINEAR_DIRECT"; value: what atoi() of the
+ * variable would give.  trtamd_test_reset_tuning returns the switch to the environment's (or the default) value.
+ * An unknown name returns TRTAMD_STATUS_BAD_PARAM. */
+TRTAMD_API int trtamd_test_set_tuning(char const* name, int32_t value);
+TRTAMD_API int trtamd_test_reset_tuning(char const* name);
+
 #ifdef __cplusplus
 }
 #endif

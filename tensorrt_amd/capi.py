@@ -107,6 +107,9 @@ _SIGS = {
     "trtamd_unfused_mha_workspace_size": (C.c_size_t, [i32, i32, i32, i32]),
     "trtamd_unfused_mha": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p, c_p]),
     "trtamd_unfused_mha_static_capacity": (C.c_size_t, []),
+    "trtamd_unfused_mha_static_prepare": (C.c_int, []),
+    "trtamd_test_set_tuning": (C.c_int, [C.c_char_p, i32]),
+    "trtamd_test_reset_tuning": (C.c_int, [C.c_char_p]),
     "trtamd_unfused_mha_static": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p]),
     "trtamd_fused_mha_run": (C.c_int, [c_p, i32, C.POINTER(FmhaParams)]),
     "trtamd_fused_mha_run_debug": (C.c_int, [c_p, i32, C.POINTER(FmhaParams), c_p, c_p]),
@@ -130,7 +133,7 @@ _SIGS = {
 }
 
 # Entry points declared in include/trtamd_test_hooks.h (test-only).
-TEST_HOOK_SYMBOLS = ["trtamd_fused_mha_run_debug"]
+TEST_HOOK_SYMBOLS = ["trtamd_fused_mha_run_debug", "trtamd_test_set_tuning", "trtamd_test_reset_tuning"]
 # Entry points declared in include/trtamd_bert_kernels.h are the rest of the table.
 # Entry points declared in include/trtamd_encoder_ops.h.
 ENCODER_OPS_SYMBOLS = ["trtamd_int8_linear", "trtamd_fp16_linear", "trtamd_int8_linear_to_interleaved", "trtamd_int8_interleaved_to_linear",

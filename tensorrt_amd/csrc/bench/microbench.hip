@@ -93,6 +93,16 @@ enum ValuOp
     OP_MAX3 = 4,
     OP_CVT_PK_U8 = 5,
     OP_SOFTMAX_MIX = 6, // fma, exp, add, fma per element: the inner sequence of the attention kernel
+    OP_MAX3_F32 = 7,
+    OP_MAX_F32 = 8,
+    OP_MUL = 9,
+    OP_LSHL_OR = 10,
+    OP_CVT_F32_I32 = 11,
+    OP_CVT_F32_BYTE = 12, // v_cvt_f32_ubyte0
+    OP_DOT4 = 13,         // v_dot4_i32_i8
+    OP_RCP = 14,
+    OP_MED3_F32 = 15,
+    OP_ADD_U32 = 16,
 };
 
 template <int OP>
@@ -137,6 +147,46 @@ __global__ __launch_bounds__(kThreads) void valu_kernel(int32_t const* src, int3
             else if (OP == OP_CVT_PK_U8)
             {
                 a[i] = __uint_as_float(__builtin_amdgcn_cvt_pk_u8_f32(a[i], 1, __float_as_uint(a[(i + 1) & 7])));
+            }
+            else if (OP == OP_MAX3_F32)
+            {
+                asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(a[i]) : "v"(a[(i + 1) & 7]), "v"(a[(i + 2) & 7]));
+            }
+            else if (OP == OP_MAX_F32)
+            {
+                asm volatile("v_max_f32 %0, %0, %1" : "+v"(a[i]) : "v"(a[(i + 1) & 7]));
+            }
+            else if (OP == OP_MUL)
+            {
+                asm volatile("v_mul_f32 %0, %0, %1" : "+v"(a[i]) : "v"(c));
+            }
+            else if (OP == OP_LSHL_OR)
+            {
+                asm volatile("v_lshl_or_b32 %0, %0, 8, %1" : "+v"(a[i]) : "v"(a[(i + 1) & 7]));
+            }
+            else if (OP == OP_CVT_F32_I32)
+            {
+                asm volatile("v_cvt_f32_i32 %0, %0" : "+v"(a[i]));
+            }
+            else if (OP == OP_CVT_F32_BYTE)
+            {
+                asm volatile("v_cvt_f32_ubyte0 %0, %0" : "+v"(a[i]));
+            }
+            else if (OP == OP_DOT4)
+            {
+                asm volatile("v_dot4_i32_i8 %0, %1, %2, %0" : "+v"(a[i]) : "v"(a[(i + 1) & 7]), "v"(c));
+            }
+            else if (OP == OP_RCP)
+            {
+                asm volatile("v_rcp_f32 %0, %0" : "+v"(a[i]));
+            }
+            else if (OP == OP_MED3_F32)
+            {
+                asm volatile("v_med3_f32 %0, %0, %1, %2" : "+v"(a[i]) : "v"(c), "v"(a[(i + 1) & 7]));
+            }
+            else if (OP == OP_ADD_U32)
+            {
+                asm volatile("v_add_u32 %0, %0, %1" : "+v"(a[i]) : "v"(a[(i + 1) & 7]));
             }
             else
             {
@@ -410,6 +460,8 @@ MB_API float trtamd_microbench_valu(int op, int blocks, int iters, int32_t const
             5);                                                                                                        \
     }
     MB_OP(OP_FMA) MB_OP(OP_EXP) MB_OP(OP_ADD) MB_OP(OP_PERM) MB_OP(OP_MAX3) MB_OP(OP_CVT_PK_U8) MB_OP(OP_SOFTMAX_MIX)
+    MB_OP(OP_MAX3_F32) MB_OP(OP_MAX_F32) MB_OP(OP_MUL) MB_OP(OP_LSHL_OR) MB_OP(OP_CVT_F32_I32) MB_OP(OP_CVT_F32_BYTE)
+    MB_OP(OP_DOT4) MB_OP(OP_RCP) MB_OP(OP_MED3_F32) MB_OP(OP_ADD_U32)
 #undef MB_OP
     return -1.f;
 }

@@ -1,14 +1,67 @@
-// Library-wide state of the C-ABI layer: version and the per-thread error text.
+// Library-wide state of the C-ABI layer: version, the per-thread error text and the tuning switches.
 #include "host_utils.hpp"
 
+#include "trtamd_test_hooks.h"
+
+#include <atomic>
+#include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 namespace trtamd
 {
 namespace
 {
 thread_local char gLastError[512] = "";
+
+struct TuningEntry
+{
+    char const* name;
+    int fallback;
+};
+constexpr TuningEntry kTuning[(int) Tuning::kCount] = {
+    {"TRTAMD_LINEAR_PARTIAL_ROUND", 50}, {"TRTAMD_LINEAR_PERSISTENT", 1}, {"TRTAMD_LINEAR_DIRECT", 1},
+    {"TRTAMD_FMHA_GENERIC", 0}, {"TRTAMD_FMHA_QSPLIT", 0}, {"TRTAMD_FMHA_RANKED", -1}, {"TRTAMD_UNFUSED_SPLIT", 0},
+};
+constexpr int kUnset = INT32_MIN;
+std::atomic<int> gTuningOverride[(int) Tuning::kCount];
+std::atomic<int> gTuningEnv[(int) Tuning::kCount];
+std::once_flag gTuningOnce;
+
+void read_tuning_env()
+{
+    for (int i = 0; i < (int) Tuning::kCount; ++i)
+    {
+        char const* e = getenv(kTuning[i].name);
+        gTuningEnv[i].store(e ? atoi(e) : kTuning[i].fallback, std::memory_order_relaxed);
+        gTuningOverride[i].store(kUnset, std::memory_order_relaxed);
+    }
 }
+} // namespace
+
+int tuning(Tuning which)
+{
+    std::call_once(gTuningOnce, read_tuning_env);
+    int const o = gTuningOverride[(int) which].load(std::memory_order_relaxed);
+    return o != kUnset ? o : gTuningEnv[(int) which].load(std::memory_order_relaxed);
+}
+
+namespace
+{
+int set_tuning(char const* name, int value, bool set)
+{
+    std::call_once(gTuningOnce, read_tuning_env);
+    for (int i = 0; name && i < (int) Tuning::kCount; ++i)
+    {
+        if (strcmp(name, kTuning[i].name) == 0)
+        {
+            gTuningOverride[i].store(set ? value : kUnset, std::memory_order_relaxed);
+            return TRTAMD_STATUS_SUCCESS;
+        }
+    }
+    return set_error(TRTAMD_STATUS_BAD_PARAM, "unknown tuning switch: %s", name ? name : "(null)");
+}
+} // namespace
 
 int set_error(int status, char const* fmt, ...)
 {
@@ -19,6 +72,16 @@ int set_error(int status, char const* fmt, ...)
     return status;
 }
 } // namespace trtamd
+
+extern "C" int trtamd_test_set_tuning(char const* name, int32_t value)
+{
+    return trtamd::set_tuning(name, value, true);
+}
+
+extern "C" int trtamd_test_reset_tuning(char const* name)
+{
+    return trtamd::set_tuning(name, 0, false);
+}
 
 extern "C" int trtamd_version(void)
 {

@@ -1695,10 +1695,7 @@ int run_i8(hipStream_t stream, FmhaArgs const& a, bool interleaved)
     int const kt = pick_kt(a.S);
     // keys are a valid prefix (cu_seqlens, or no mask) and probabilities cannot leave the INT8 range:
     // the kernel specialised on the number of key blocks serves the launch
-    static int const noFast = [] {
-        char const* e = getenv("TRTAMD_FMHA_GENERIC");
-        return e ? atoi(e) : 0;
-    }();
+    int const noFast = tuning(Tuning::kFmhaGeneric);
     if (a.packedMask == nullptr && !a.clampP && !noFast)
     {
 #define TRTAMD_I8P(KT)                                                                                                 \
@@ -1743,10 +1740,7 @@ template <bool DEBUG>
 int run_f16(hipStream_t stream, FmhaArgs const& a)
 {
     int const kt = pick_kt(a.S);
-    static int const noFast = [] {
-        char const* e = getenv("TRTAMD_FMHA_GENERIC");
-        return e ? atoi(e) : 0;
-    }();
+    int const noFast = tuning(Tuning::kFmhaGeneric);
     if (a.packedMask == nullptr && !noFast)
     {
 #define TRTAMD_F16P(KT)                                                                                                \
@@ -1883,10 +1877,7 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
         }
         a.qSplit = std::min(split, maxSplit);
         // tuning override: TRTAMD_FMHA_QSPLIT=<n> forces the number of workgroups per head
-        static int const forced = [] {
-            char const* e = getenv("TRTAMD_FMHA_QSPLIT");
-            return e ? atoi(e) : 0;
-        }();
+        int const forced = tuning(Tuning::kFmhaQsplit);
         if (forced > 0)
         {
             a.qSplit = std::min(forced, maxSplit);
@@ -1903,10 +1894,7 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
         int64_t const perCu = std::max<int64_t>(1, std::min<int64_t>(dataType == 2 ? 3 : 2, (160 * 1024) / std::max<int64_t>(lds, 1)));
         a.ranked = (int64_t) a.B * a.N * a.qSplit > perCu * 256 ? 1 : 0;
         // tuning override: TRTAMD_FMHA_RANKED=0 / 1 forces natural order / the longest-first order
-        static int const forcedRank = [] {
-            char const* e = getenv("TRTAMD_FMHA_RANKED");
-            return e ? atoi(e) : -1;
-        }();
+        int const forcedRank = tuning(Tuning::kFmhaRanked);
         if (forcedRank >= 0)
         {
             a.ranked = forcedRank ? 1 : 0;

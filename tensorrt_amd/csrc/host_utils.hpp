@@ -37,6 +37,22 @@ inline bool aligned16(void const* p)
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
 
+// Tuning switches: kernel variants other than the default choice, selectable with an environment variable (read once
+// per process, at the first use of the switch) or, from the tests, with trtamd_test_set_tuning (which wins).  A
+// launcher reads a switch once per call and hands the decision down, so a change between two reads cannot split a call.
+enum class Tuning : int
+{
+    kLinearPartialRound = 0, // TRTAMD_LINEAR_PARTIAL_ROUND=<percent>, default 50
+    kLinearPersistent,       // TRTAMD_LINEAR_PERSISTENT=0/1, default 1
+    kLinearDirect,           // TRTAMD_LINEAR_DIRECT=0/1, default 1
+    kFmhaGeneric,            // TRTAMD_FMHA_GENERIC=0/1, default 0
+    kFmhaQsplit,             // TRTAMD_FMHA_QSPLIT=<n>, default 0 (chosen from the launch size)
+    kFmhaRanked,             // TRTAMD_FMHA_RANKED=0/1, default -1 (chosen from the launch size)
+    kUnfusedSplit,           // TRTAMD_UNFUSED_SPLIT=0/1, default 0
+    kCount
+};
+int tuning(Tuning which);
+
 template <typename T>
 constexpr T ceil_div(T a, T b)
 {

@@ -672,11 +672,11 @@ __device__ __forceinline__ void linear_tile_run(
 //   per row, 64 contiguous bytes of it); in LDS the 16-byte chunk c of row r sits at chunk c ^ (r / 4), which makes
 //   the fragment reads (16 rows x one chunk per 16 lanes) conflict-free; fragment (block, ks) takes chunks 2 ks and
 //   2 ks + 1 of the block's two units.
-template <bool IL, bool IL_OUT, int EPI, int KS, typename Origin>
+template <bool IL, bool IL_OUT, int EPI, typename Origin>
 __device__ __forceinline__ void linear_tile_run_dma(
     LinearArgs const& p, int const count, Origin origin, uint8_t* __restrict__ lds, float* sScale)
 {
-    static_assert(KS == 2 || (KS == 1 && IL), "32-byte stages are built for the interleaved layout only");
+    constexpr int KS = 2; // k-halves of 32 bytes per stage
     constexpr int WN = 4, MT = 4, NT = 2, NWAVES = 8;
     constexpr int AF = (kBigTile / 32) * KS;   // 1 KB fragments per operand and stage: KS k-halves of 32 bytes per row block
     constexpr int BF = (kBigTile / 32) * KS;
@@ -712,7 +712,7 @@ __device__ __forceinline__ void linear_tile_run_dma(
         laneOff = (uint32_t) rr * (uint32_t) p.K + chunk * 16u;
     }
     auto unit_base = [&](int u, int row0, int R) -> uint32_t {
-        int const rb = KS == 2 ? u >> 1 : u, sel = KS == 2 ? u & 1 : 0;
+        int const rb = u >> 1, sel = u & 1;
         uint32_t const b = IL ? ((uint32_t) sel * (uint32_t) R + (uint32_t) (row0 + rb * 32)) * 32u
                               : (uint32_t) (row0 + rb * 32 + sel * 16) * (uint32_t) p.K;
         return (uint32_t) __builtin_amdgcn_readfirstlane((int) b);
@@ -988,10 +988,10 @@ __global__ __launch_bounds__(512) void int8_linear_persistent_kernel(LinearArgs 
 }
 
 // The persistent tile plan with direct-to-LDS loads for the 256 x 256 tiles.
-template <bool IL, bool IL_OUT, int EPI, int KS = 2>
+template <bool IL, bool IL_OUT, int EPI>
 __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[4 * 2 * (kBig / 32) * KS * 1024];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[4 * 2 * (kBig / 32) * 2 * 1024];
     __shared__ __attribute__((aligned(16))) float sScale[2 * 2 * kBig];
     if ((int) blockIdx.x < p.persist)
     {
@@ -1004,7 +1004,7 @@ __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p
             n0 = (int) (pan * pw + rem % pw) * kBig;
             t0 = (int) (rem / pw) * kBig;
         };
-        linear_tile_run_dma<IL, IL_OUT, EPI, KS>(p, count, origin, lds, sScale);
+        linear_tile_run_dma<IL, IL_OUT, EPI>(p, count, origin, lds, sScale);
     }
     else
     {
@@ -1041,10 +1041,7 @@ int launch_shape(hipStream_t stream, LinearArgs a)
     int const cus = num_cus();
     // ... plus a last partial round when it would occupy more than `partial` per cent of the CUs: in 128 x 128
     // tiles that remainder needs three rounds or more, which take longer than one round of large tiles
-    static int const partial = [] {
-        char const* e = getenv("TRTAMD_LINEAR_PARTIAL_ROUND");
-        return e ? atoi(e) : 50;
-    }();
+    int const partial = tuning(Tuning::kLinearPartialRound);
     int64_t roundedTiles = (bigTiles / cus) * cus;
     if ((bigTiles - roundedTiles) * 100 > (int64_t) partial * cus)
     {
@@ -1067,33 +1064,14 @@ int launch_shape(hipStream_t stream, LinearArgs a)
     {
         return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "int8_linear: too many tiles");
     }
-    static int const persistent = [] {
-        char const* e = getenv("TRTAMD_LINEAR_PERSISTENT");
-        return e ? atoi(e) : 1;
-    }();
+    int const persistent = tuning(Tuning::kLinearPersistent);
     if (persistent && a.K % 128 == 0)
     {
         a.persist = a.mainTiles < cus ? a.mainTiles : cus;
         int64_t const pgrid = grid - a.mainTiles + a.persist;
-        static int const direct = [] {
-            char const* e = getenv("TRTAMD_LINEAR_DIRECT");
-            return e ? atoi(e) : 1;
-        }();
+        int const direct = tuning(Tuning::kLinearDirect);
         if constexpr (IL_W == IL_IN && (EPI == kAFFINE || EPI == kGELU || EPI == kF16_AFFINE || EPI == kF16_GELU))
         {
-            static int const stage32 = [] {
-                char const* e = getenv("TRTAMD_LINEAR_STAGE32");
-                return e ? atoi(e) : 0;
-            }();
-            if constexpr (IL_W && (EPI == kAFFINE || EPI == kGELU))
-            {
-                if (stage32 && direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
-                {
-                    hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI, 1>), dim3((uint32_t) pgrid), dim3(512), 0,
-                        stream, a);
-                    return check_launch("int8_linear_dma_kernel(32-byte stages)");
-                }
-            }
             if (direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
             {
                 hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0, stream,

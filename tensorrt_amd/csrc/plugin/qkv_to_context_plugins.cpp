@@ -116,12 +116,16 @@ bool fusedV1Valid(DataType type, int32_t headSize, int32_t S)
 }
 
 // What creating a fused runner does in the reference (getXMMAKernels / getXMMAKernelsV2 load every kernel and raise
-// its shared-memory limit, fused_multihead_attention.h:63-147): afterwards enqueue only launches.
-void prepareFusedKernels()
+// its shared-memory limit, fused_multihead_attention.h:63-147): afterwards enqueue only launches.  Only the types the
+// fused kernels serve ask for it, and a failure is logged, not thrown: a launch raises the limit of its own kernel
+// again if it has to, and an object that never launches a fused kernel must not fail to exist over them.
+void prepareFusedKernels(DataType type)
 {
-    if (deviceAvailable())
+    if ((type == DataType::kHALF || type == DataType::kINT8) && deviceAvailable()
+        && trtamd_fused_mha_prepare() != TRTAMD_STATUS_SUCCESS)
     {
-        checkKernelStatus(trtamd_fused_mha_prepare(), "fused attention kernels");
+        logMessage(ILogger::Severity::kWARNING,
+            std::string("fused attention kernels could not be prepared ahead of the first enqueue: ") + trtamd_last_error());
     }
 }
 
@@ -176,7 +180,7 @@ public:
     {
         mSM = getSmVersion();
         mUnfused.unfused = true;
-        prepareFusedKernels();
+        prepareFusedKernels(mType);
     }
 
     // runtime-phase constructor (deserialised engine)
@@ -589,7 +593,7 @@ public:
             TRTAMD_VALIDATE(mType != DataType::kINT8);
         }
         mRunner.unfused = !varSeqlen;
-        prepareFusedKernels();
+        prepareFusedKernels(mType);
     }
 
     QkvToContextVarSeqlenPlugin(std::string const& name, int32_t S, int32_t B, DataType type, int32_t hiddenSize,
@@ -962,7 +966,7 @@ public:
         , mCtxScale(ctxScale)
     {
         mSM = getSmVersion();
-        prepareFusedKernels();
+        prepareFusedKernels(DataType::kINT8);
     }
 
 protected:

@@ -295,7 +295,8 @@ public:
     int enqueueConcurrent(trtamd_encoder_batch const* parts, int32_t count, hipStream_t stream)
     {
         requireComplete();
-        TRTAMD_VALIDATE_MSG(parts != nullptr && count >= 1 && count <= contexts(),
+        TRTAMD_VALIDATE_MSG(parts != nullptr && count >= 1, "at least one part is required");
+        TRTAMD_VALIDATE_MSG(count <= contexts(),
             "more parts than reserved execution contexts (trtamd_encoder_reserve_contexts)");
         std::vector<Pass> passes;
         passes.reserve(static_cast<size_t>(count));
@@ -304,16 +305,12 @@ public:
             Context& c = mContexts[static_cast<size_t>(i)];
             passes.emplace_back(*this, c, parts[i], i == 0 ? stream : c.side.stream);
         }
-        // arguments are checked (above) before anything is recorded, so that a refused call leaves no stream forked
-        for (int32_t i = 1; i < count; ++i)
-        {
-            Side const& sd = mContexts[static_cast<size_t>(i)].side;
-            TRTAMD_VALIDATE(hipEventRecord(sd.fork, stream) == hipSuccess);
-            TRTAMD_VALIDATE(hipStreamWaitEvent(sd.stream, sd.fork, 0) == hipSuccess);
-        }
+        // arguments are checked (above) before anything is recorded, so that a refused call leaves no stream forked;
+        // if forking fails half way, the streams forked so far are joined again before the error leaves
+        int32_t forked = 1;
         auto join = [&] {
             bool ok = true;
-            for (int32_t i = 1; i < count; ++i)
+            for (int32_t i = 1; i < forked; ++i)
             {
                 Side const& sd = mContexts[static_cast<size_t>(i)].side;
                 ok = hipEventRecord(sd.join, sd.stream) == hipSuccess && ok;
@@ -323,6 +320,13 @@ public:
         };
         try
         {
+            for (int32_t i = 1; i < count; ++i)
+            {
+                Side const& sd = mContexts[static_cast<size_t>(i)].side;
+                TRTAMD_VALIDATE(hipEventRecord(sd.fork, stream) == hipSuccess);
+                TRTAMD_VALIDATE(hipStreamWaitEvent(sd.stream, sd.fork, 0) == hipSuccess);
+                forked = i + 1;
+            }
             for (Pass& p : passes)
             {
                 p.embed();

@@ -929,24 +929,19 @@ int launch_attention_in_registers(hipStream_t stream, int32_t S, int32_t B, int3
     return check_launch("attention_in_registers_kernel");
 }
 
-// TRTAMD_UNFUSED_SPLIT=1 keeps every shape on the three kernels with the score matrices in the workspace.
-bool one_launch_allowed()
-{
-    char const* e = getenv("TRTAMD_UNFUSED_SPLIT");
-    return !(e && e[0] == '1');
-}
-
-// Whether a shape runs in the one-launch kernel (and so needs no score matrices).
+// Whether a shape runs in the one-launch kernel (and so needs no score matrices).  The tuning switch
+// TRTAMD_UNFUSED_SPLIT=1 keeps every shape on the three kernels with the score matrices in the workspace; an entry
+// point asks once per call and hands the answer down.
 bool scores_in_registers(int32_t S, int32_t d)
 {
-    return S <= kRegMaxS && d <= kRegMaxD && one_launch_allowed();
+    return S <= kRegMaxS && d <= kRegMaxD && tuning(Tuning::kUnfusedSplit) == 0;
 }
 
 template <typename T>
 int unfused_mha(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, T const* qkv, int32_t const* maskIdx,
-    T* output, void* workspace)
+    T* output, void* workspace, bool const inRegisters)
 {
-    if (scores_in_registers(S, d))
+    if (inRegisters)
     {
         return d <= 64 ? launch_attention_in_registers<T, 64>(stream, S, B, N, d, qkv, maskIdx, output)
                        : launch_attention_in_registers<T, 128>(stream, S, B, N, d, qkv, maskIdx, output);
@@ -1038,6 +1033,34 @@ extern "C" size_t trtamd_unfused_mha_workspace_size(int32_t type, int32_t S, int
     return 2UL * word * (size_t) S * (size_t) S * (size_t) B * (size_t) N;
 }
 
+namespace trtamd
+{
+namespace
+{
+// Both entry points of the unfused attention after their own checks; inRegisters: the caller's one reading of
+// scores_in_registers for this call.
+int run_unfused(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d, void const* qkv,
+    int32_t const* maskIdx, void* output, void* workspace, bool const inRegisters)
+{
+    if ((int64_t) B * N > 65535)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: B*N = %lld exceeds 65535", (long long) B * N);
+    }
+    if (!qkv || !output || !workspace)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: null pointer (workspace is required)");
+    }
+    if (type == 0)
+    {
+        return unfused_mha<float>(as_stream(stream), S, B, N, d, static_cast<float const*>(qkv), maskIdx,
+            static_cast<float*>(output), workspace, inRegisters);
+    }
+    return unfused_mha<f16>(as_stream(stream), S, B, N, d, static_cast<f16 const*>(qkv), maskIdx,
+        static_cast<f16*>(output), workspace, inRegisters);
+}
+} // namespace
+} // namespace trtamd
+
 extern "C" int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
     void const* qkv, int32_t const* maskIdx, void* output, void* workspace)
 {
@@ -1050,26 +1073,19 @@ extern "C" int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
     {
         return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
     }
-    if ((int64_t) B * N > 65535)
-    {
-        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: B*N = %lld exceeds 65535", (long long) B * N);
-    }
-    if (!qkv || !output || !workspace)
-    {
-        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: null pointer (workspace is required)");
-    }
-    if (type == 0)
-    {
-        return unfused_mha<float>(as_stream(stream), S, B, N, d, static_cast<float const*>(qkv), maskIdx,
-            static_cast<float*>(output), workspace);
-    }
-    return unfused_mha<f16>(as_stream(stream), S, B, N, d, static_cast<f16 const*>(qkv), maskIdx,
-        static_cast<f16*>(output), workspace);
+    return trtamd::run_unfused(stream, type, S, B, N, d, qkv, maskIdx, output, workspace,
+        trtamd::scores_in_registers(S, d));
 }
 
 extern "C" size_t trtamd_unfused_mha_static_capacity(void)
 {
     return kStaticScratchBytes;
+}
+
+extern "C" int trtamd_unfused_mha_static_prepare(void)
+{
+    void* ws = nullptr;
+    return static_scratch(&ws);
 }
 
 extern "C" int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
@@ -1102,7 +1118,7 @@ extern "C" int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, i
     }
     // every score the second and third kernel read was written by the kernel before it in this call: nothing in
     // the array has to start at zero, and what the previous call left there is never read
-    return trtamd_unfused_mha(stream, type, S, B, N, d, qkv, maskIdx, output, ws);
+    return trtamd::run_unfused(stream, type, S, B, N, d, qkv, maskIdx, output, ws, inRegisters);
 }
 
 extern "C" int trtamd_zero_padding_2d(

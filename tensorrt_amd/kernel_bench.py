@@ -73,7 +73,8 @@ def microbench(torch, cus: int = 256) -> dict:
     res["v_mfma_i32_16x16x64_i8.one_wave_per_simd_one_accumulator.TOP/s"] = round(
         cus * 4 * iters * 2 * 16 * 16 * 64 / (ms * 1e-3) / 1e12, 1)
     names = ["v_fma_f32", "v_exp_f32", "v_add_f32", "v_perm_b32", "v_max3_i32", "v_cvt_pk_u8_f32",
-             "fma+exp+add+fma (softmax inner sequence)"]
+             "fma+exp+add+fma (softmax inner sequence)", "v_max3_f32", "v_max_f32", "v_mul_f32", "v_lshl_or_b32",
+             "v_cvt_f32_i32", "v_cvt_f32_ubyte0", "v_dot4_i32_i8", "v_rcp_f32", "v_med3_f32", "v_add_u32"]
     valu = {}
     mhz = []
     for op, name in enumerate(names):

@@ -82,16 +82,18 @@ def _run_unfused(api, dt, S, B, N, d, qkv, lens):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
 @pytest.mark.parametrize("S,B,N,d", [(384, 3, 4, 64), (200, 2, 2, 128), (97, 2, 3, 40), (512, 1, 2, 32)])
-def test_one_launch_against_the_three_kernels(api, monkeypatch, dt, S, B, N, d):
+def test_one_launch_against_the_three_kernels(api, dt, S, B, N, d):
     """Both routes round scores and probabilities to the storage type at the same places; what is left between them
     is the order of the binary32 sums."""
     r = rng(800 + S + d)
     qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
     lens = r.integers(1, S + 1, B).astype(np.int32)
     lens[0] = S
-    monkeypatch.setenv("TRTAMD_UNFUSED_SPLIT", "1")
-    split = _run_unfused(api, dt, S, B, N, d, qkv, lens)
-    monkeypatch.setenv("TRTAMD_UNFUSED_SPLIT", "0")
+    api.check(api.test_set_tuning(b"TRTAMD_UNFUSED_SPLIT", 1))
+    try:
+        split = _run_unfused(api, dt, S, B, N, d, qkv, lens)
+    finally:
+        api.check(api.test_reset_tuning(b"TRTAMD_UNFUSED_SPLIT"))
     one = _run_unfused(api, dt, S, B, N, d, qkv, lens)
     tol = dict(atol=2e-6, rtol=2e-5) if dt == np.float32 else dict(atol=1e-3, rtol=2e-3)
     assert_fp_close(one, split, what="one launch vs three kernels", **tol)

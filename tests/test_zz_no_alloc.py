@@ -72,3 +72,39 @@ def test_sizes_beyond_the_array_are_refused(api):
     assert api.unfused_mha_workspace_size(1, 512, 2, 16) == cap
     assert api.unfused_mha_static(stream(), 5, 16, 1, 1, 8, ptr(x), 0, ptr(x)) == 3      # INT8 etc.: as the other entry
     assert api.unfused_mha_static(stream(), 0, 0, 1, 1, 8, ptr(x), 0, ptr(x)) == 2
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_captured_in_a_graph_and_no_device_memory_taken(api, dt):
+    """The entry point under stream capture (the array's address looked up beforehand): every replay, with eager work
+    between the replays, gives the eager result, and the calls leave the amount of free device memory as it was."""
+    import torch
+    S, B, N, d = 640, 2, 3, 64                  # scores go through the array
+    r = rng(331)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
+    lens = np.array([S, 300], np.int32)
+    type_id = 0 if dt == np.float32 else 1
+    d_qkv, d_len = dev(qkv), dev(lens)
+    eager = dev_empty((S, B, N * d), dt, fill=0)
+    got = dev_empty((S, B, N * d), dt, fill=0)
+    api.check(api.unfused_mha_static_prepare())
+    api.check(api.unfused_mha_static(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(eager)))
+    sync()
+    free_before = torch.cuda.mem_get_info()[0]
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            api.check(api.unfused_mha_static(side.cuda_stream, type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(got)))
+    u = np.uint32 if dt == np.float32 else np.uint16
+    for replay in range(3):
+        got.zero_()
+        # eager work of the same entry point on another problem between the replays: it overwrites the array
+        _both(api, dt, 520, 1, 2, 32, seed=340 + replay)
+        graph.replay()
+        sync()
+        assert np.array_equal(host(got).view(u), host(eager).view(u)), f"replay {replay} differs from the eager call"
+    api.check(api.unfused_mha_static(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(got)))
+    sync()
+    del graph
+    assert torch.cuda.mem_get_info()[0] >= free_before, "the calls took device memory"
