@@ -90,7 +90,12 @@ def test_captured_in_a_graph_and_no_device_memory_taken(api, dt):
     api.check(api.unfused_mha_static_prepare())
     api.check(api.unfused_mha_static(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(eager)))
     sync()
+    # no allocation by anyone between the two readings: only calls of the entry point
     free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        api.check(api.unfused_mha_static(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(got)))
+    sync()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the calls changed the amount of free device memory"
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
@@ -104,7 +109,4 @@ def test_captured_in_a_graph_and_no_device_memory_taken(api, dt):
         graph.replay()
         sync()
         assert np.array_equal(host(got).view(u), host(eager).view(u)), f"replay {replay} differs from the eager call"
-    api.check(api.unfused_mha_static(stream(), type_id, S, B, N, d, ptr(d_qkv), ptr(d_len), ptr(got)))
-    sync()
     del graph
-    assert torch.cuda.mem_get_info()[0] >= free_before, "the calls took device memory"
