@@ -148,8 +148,8 @@ TRTAMD_API int trtamd_scaled_softmax_fp16(trtamd_stream_t stream, int32_t ld, in
 /* UnfusedMHARunner::run  plugin/bertQKVToContextPlugin/mhaRunner.cu:527-601 with the geometry of
  * MHARunner::setup (plugin/bertQKVToContextPlugin/mhaRunner.h:62-83): qkv [S,B,N,3,d], output
  * [S,B,N,d], maskIdx [B] or NULL, workspace of trtamd_unfused_mha_workspace_size bytes (the reference's two S x S
- * matrices per batch and head; required, and written only for S > 512 or d > 128 — smaller shapes run in one launch
- * that keeps a query's scores in registers).
+ * matrices per batch and head; required, and written only for head sizes d > 128 — other shapes run in one launch
+ * that never stores a score: up to 512 keys a query's scores stay in registers, beyond that the keys are walked twice).
  * type: 0 = fp32, 1 = fp16 (nvinfer1::DataType values). */
 TRTAMD_API size_t trtamd_unfused_mha_workspace_size(int32_t type, int32_t S, int32_t B, int32_t N);
 TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
@@ -164,8 +164,8 @@ TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
  * trtamd_unfused_mha_static on the device.  A problem whose trtamd_unfused_mha_workspace_size exceeds the capacity is
  * refused with TRTAMD_STATUS_NOT_SUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU
  * (different streams) race; calls on one stream, or ordered by events, are safe.  The array is used, and the limit
- * applies, for the shapes whose scores go through memory (S > 512 or d > 128); smaller shapes keep their scores in
- * registers, touch nothing of the array and are accepted at any batch size. */
+ * applies, for the shapes whose scores go through memory (head sizes d > 128); all others run in one launch that
+ * stores no score, touch nothing of the array and are accepted at any size. */
 TRTAMD_API size_t trtamd_unfused_mha_static_capacity(void);
 TRTAMD_API int trtamd_unfused_mha_static_prepare(void);
 TRTAMD_API int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N,

@@ -498,7 +498,7 @@ int can_vectorise(T const* base, GemmOperand const& o)
 // ------------------------------------------------------------------------------------------
 constexpr int kRegQueries = 64; // queries per workgroup
 constexpr int kRegKeys = 64;    // keys per LDS stage
-constexpr int kRegMaxS = 512;
+constexpr int kRegMaxS = 512;  // keys whose scores one lane can hold (32 tiles); longer sequences walk the keys twice
 constexpr int kRegMaxD = 128;
 
 template <typename T, int DP>
@@ -887,6 +887,341 @@ __global__ __launch_bounds__(kBlock, (reg_waves<T, DP, NT>())) void attention_in
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// One launch for sequences beyond 512 keys (head size <= 128): the scores of a query no longer fit in registers, so
+// the keys are walked twice in stages of 64.  The first pass computes the scores of a stage, keeps each lane's running
+// maximum and the sum of exponentials relative to it (rescaled when the maximum moves) and drops the scores; the four
+// lane groups of a query are combined at the end.  The second pass computes the scores again, forms the
+// probabilities with the row's maximum and sum now known, rounds them to T as the softmax of the three-kernel path
+// stores them, and multiplies them with V.  Same roundings as the kernel above (scores to T, probabilities to T,
+// binary32 accumulation); the only difference to it is the order of the binary32 sum of exponentials.  K is read
+// twice and the first product is computed twice; no score goes to memory.
+// Work split, operand layouts in LDS and fragment orders are those of attention_in_registers_kernel; K and V each
+// have one LDS stage and are fetched into registers D stages ahead.
+// ------------------------------------------------------------------------------------------
+template <typename T, int DP>
+__global__ __launch_bounds__(kBlock, 2) void attention_two_pass_kernel(int const S, int const heads, int const d,
+    int const strips, float const w, T const* __restrict__ qkv, int64_t const ldQKV,
+    int32_t const* __restrict__ maskIdx, T* __restrict__ out, int64_t const ldOut, int const vecIn, int const vecOut)
+{
+    using L = RegLds<T, DP>;
+    using Frag = typename RegFrag<T>::type;
+    constexpr int V = L::V;
+    constexpr int kPieces = DP / V;
+    constexpr int kSteps = DP / (4 * V);
+    constexpr int kDimTiles = DP / 16;
+    constexpr bool kHalf = sizeof(T) == 2;
+    constexpr int NP = kRegKeys * kPieces / kBlock;
+    constexpr int D = kHalf ? (DP <= 64 ? 3 : 2) : 1; // stages in flight ahead of the one in LDS
+    __shared__ __attribute__((aligned(16))) T ldsK[kRegKeys * L::kPitchK];
+    __shared__ __attribute__((aligned(16))) T ldsV[L::kElemsV];
+
+    int const strip = blockIdx.x % strips;
+    int const z = blockIdx.x / strips;
+    int const lane = threadIdx.x & (kWaveSize - 1);
+    int const wave = threadIdx.x >> 6;
+    int const n = lane & 15, g = lane >> 4;
+    int const query = strip * kRegQueries + wave * 16 + n;
+    bool const vec = vecIn != 0;
+    T const* const qp = qkv + (int64_t) z * 3 * d;
+    T const* const kp = qp + d;
+    T const* const vp = qp + 2 * d;
+    int valid = S;
+    if (maskIdx)
+    {
+        valid = max(0, min(S, maskIdx[z / heads]));
+    }
+    int const nChunks = (valid + kRegKeys - 1) / kRegKeys;
+
+    Frag qf[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t)
+    {
+        qf[t] = load_piece<T>(qp + (int64_t) query * ldQKV, 4 * V * t + V * g, d, query < S, vec);
+    }
+    auto fetch_k = [&](Frag(&dst)[NP], int const c)
+    {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+        {
+            int const p = threadIdx.x + it * kBlock;
+            int const gk = c * kRegKeys + p / kPieces;
+            dst[it] = load_piece<T>(kp + (int64_t) gk * ldQKV, (p % kPieces) * V, d, gk < S, vec);
+        }
+    };
+    auto fetch_v = [&](Frag(&dst)[NP], int const c)
+    {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+        {
+            int const p = threadIdx.x + it * kBlock;
+            int const gk = c * kRegKeys + (kHalf ? p / kPieces : p % kRegKeys);
+            dst[it] = load_piece<T>(vp + (int64_t) gk * ldQKV, (kHalf ? p % kPieces : p / kRegKeys) * V, d, gk < S,
+                vec);
+        }
+    };
+    auto store_k = [&](Frag const(&src)[NP])
+    {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+        {
+            int const p = threadIdx.x + it * kBlock;
+            *reinterpret_cast<Frag*>(&ldsK[(p / kPieces) * L::kPitchK + (p % kPieces) * V]) = src[it];
+        }
+    };
+    auto store_v = [&](Frag const(&src)[NP])
+    {
+#pragma unroll
+        for (int it = 0; it < NP; ++it)
+        {
+            int const p = threadIdx.x + it * kBlock;
+            if constexpr (kHalf)
+            {
+                *reinterpret_cast<Frag*>(&ldsV[(p / kPieces) * L::kPitchV + (p % kPieces) * V]) = src[it];
+            }
+            else
+            {
+#pragma unroll
+                for (int i = 0; i < V; ++i)
+                {
+                    ldsV[((p / kRegKeys) * V + i) * L::kPitchV + p % kRegKeys] = src[it][i];
+                }
+            }
+        }
+    };
+    // the scores of the stage in ldsK, as the GEMM of the three-kernel path stores them; masked keys of the ragged
+    // tile get the most negative score, whose exponential is exactly 0
+    auto scores = [&](f32x4(&x)[4], int const c)
+    {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < kSteps; ++t)
+            {
+                if (4 * V * t < d)
+                {
+                    Frag const kf = *reinterpret_cast<Frag const*>(&ldsK[(16 * j + n) * L::kPitchK + 4 * V * t + V * g]);
+                    if constexpr (kHalf)
+                    {
+                        sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t], sc, 0, 0, 0);
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                        {
+                            sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], qf[t][i], sc, 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            if constexpr (kHalf)
+            {
+                sc = __builtin_convertvector(__builtin_convertvector(sc, f16x4), f32x4);
+            }
+            int const key0 = c * kRegKeys + 16 * j;
+            if (key0 + 16 > valid)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    sc[i] = key0 + 4 * g + i < valid ? sc[i] : -3.0e38f;
+                }
+            }
+            x[j] = sc;
+        }
+    };
+
+    float const wl2 = w * 1.4426950408889634f;
+    Frag ringK[D][NP];
+
+    // ---- first pass: row maximum and sum of exponentials -------------------------------------------------------
+    float mx = -3.0e38f, sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < D; ++u)
+    {
+        if (u < nChunks)
+        {
+            fetch_k(ringK[u], u);
+        }
+    }
+    for (int c0 = 0; c0 < nChunks; c0 += D)
+    {
+#pragma unroll
+        for (int u = 0; u < D; ++u)
+        {
+            int const c = c0 + u;
+            if (c < nChunks)
+            {
+                __syncthreads(); // the stage before this one has been read by everyone
+                store_k(ringK[u]);
+                __syncthreads();
+                if (c + D < nChunks)
+                {
+                    fetch_k(ringK[u], c + D);
+                }
+                f32x4 x[4];
+                scores(x, c);
+                float cm = mx;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    cm = fmaxf(fmaxf(cm, fmaxf(x[j][0], x[j][1])), fmaxf(x[j][2], x[j][3]));
+                }
+                // the sum so far, relative to the new maximum (a factor of exactly 1 when it did not move)
+                sum *= __builtin_amdgcn_exp2f((mx - cm) * wl2);
+                mx = cm;
+                float const nm = -cm * wl2;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        sum += __builtin_amdgcn_exp2f(fmaf(x[j][i], wl2, nm));
+                    }
+                }
+            }
+        }
+    }
+    // the four lane groups of a query hold disjoint keys: bring their sums to the common maximum and add them
+    {
+        float all = fmaxf(mx, __shfl_xor(mx, 16));
+        all = fmaxf(all, __shfl_xor(all, 32));
+        sum *= __builtin_amdgcn_exp2f((mx - all) * wl2);
+        mx = all;
+        sum += __shfl_xor(sum, 16);
+        sum += __shfl_xor(sum, 32);
+    }
+    float const nmx = -mx * wl2;
+    float const rz = 1.f / sum;
+
+    // ---- second pass: the scores again, probabilities, O^T = V^T P^T ---------------------------------------------
+    Frag ringV[D][NP];
+#pragma unroll
+    for (int u = 0; u < D; ++u)
+    {
+        if (u < nChunks)
+        {
+            fetch_k(ringK[u], u);
+            fetch_v(ringV[u], u);
+        }
+    }
+    f32x4 o[kDimTiles];
+#pragma unroll
+    for (int dt = 0; dt < kDimTiles; ++dt)
+    {
+        o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int c0 = 0; c0 < nChunks; c0 += D)
+    {
+#pragma unroll
+        for (int u = 0; u < D; ++u)
+        {
+            int const c = c0 + u;
+            if (c < nChunks)
+            {
+                __syncthreads();
+                store_k(ringK[u]);
+                store_v(ringV[u]);
+                __syncthreads();
+                if (c + D < nChunks)
+                {
+                    fetch_k(ringK[u], c + D);
+                    fetch_v(ringV[u], c + D);
+                }
+                f32x4 x[4];
+                scores(x, c);
+                typedef T Tx4 __attribute__((ext_vector_type(4)));
+                Tx4 pr[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    f32x4 e;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        e[i] = __builtin_amdgcn_exp2f(fmaf(x[j][i], wl2, nmx));
+                    }
+                    pr[j] = __builtin_convertvector(e * rz, Tx4);
+                }
+#pragma unroll
+                for (int dt = 0; dt < kDimTiles; ++dt)
+                {
+                    if (16 * dt < d)
+                    {
+                        if constexpr (kHalf)
+                        {
+#pragma unroll
+                            for (int s2 = 0; s2 < 2; ++s2)
+                            {
+                                T const* const vb
+                                    = &ldsV[(32 * s2 + 4 * g + (n >> 2)) * L::kPitchV + 16 * dt + 4 * (n & 3)];
+                                i16x4 const lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) vb);
+                                i16x4 const hi
+                                    = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*) (vb + 16 * L::kPitchV));
+                                f16x8 const vf = __builtin_bit_cast(
+                                    f16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                                f16x8 const pf
+                                    = __builtin_shufflevector(pr[2 * s2], pr[2 * s2 + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[dt], 0, 0, 0);
+                            }
+                        }
+                        else
+                        {
+                            T const* const vrow = &ldsV[(16 * dt + n) * L::kPitchV];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                            {
+                                f32x4 const vf = *reinterpret_cast<f32x4 const*>(vrow + 16 * j + 4 * g);
+#pragma unroll
+                                for (int i = 0; i < 4; ++i)
+                                {
+                                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i], pr[j][i], o[dt], 0, 0, 0);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    if (query < S)
+    {
+        T* const orow = out + (int64_t) query * ldOut + (int64_t) z * d;
+#pragma unroll
+        for (int dt = 0; dt < kDimTiles; ++dt)
+        {
+            int const d0 = 16 * dt + 4 * g;
+            T res[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                res[i] = (T) o[dt][i];
+            }
+            if (vecOut && d0 + 4 <= d)
+            {
+                typedef T Tx4 __attribute__((ext_vector_type(4)));
+                *reinterpret_cast<Tx4*>(orow + d0) = Tx4{res[0], res[1], res[2], res[3]};
+            }
+            else
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    if (d0 + i < d)
+                    {
+                        orow[d0 + i] = res[i];
+                    }
+                }
+            }
+        }
+    }
+}
+
 template <typename T, int DP>
 int launch_attention_in_registers(hipStream_t stream, int32_t S, int32_t B, int32_t N, int32_t d, T const* qkv,
     int32_t const* maskIdx, T* output)
@@ -921,20 +1256,27 @@ int launch_attention_in_registers(hipStream_t stream, int32_t S, int32_t B, int3
     {
         TRTAMD_LAUNCH_REG(24);
     }
-    else
+    else if (tiles <= 32)
     {
         TRTAMD_LAUNCH_REG(32);
+    }
+    else
+    {
+        hipLaunchKernelGGL((attention_two_pass_kernel<T, DP>), grid, block, 0, stream, S, N, d, strips, w, qkv, ldQKV,
+            maskIdx, output, ldOut, vecIn, vecOut);
+        return check_launch("attention_two_pass_kernel");
     }
 #undef TRTAMD_LAUNCH_REG
     return check_launch("attention_in_registers_kernel");
 }
 
-// Whether a shape runs in the one-launch kernel (and so needs no score matrices).  The tuning switch
+// Whether a shape runs in one of the one-launch kernels (and so needs no score matrices): every sequence length, head
+// sizes up to 128.  The tuning switch
 // TRTAMD_UNFUSED_SPLIT=1 keeps every shape on the three kernels with the score matrices in the workspace; an entry
 // point asks once per call and hands the answer down.
-bool scores_in_registers(int32_t S, int32_t d)
+bool runs_in_one_launch(int32_t S, int32_t d)
 {
-    return S <= kRegMaxS && d <= kRegMaxD && tuning(Tuning::kUnfusedSplit) == 0;
+    return d <= kRegMaxD && tuning(Tuning::kUnfusedSplit) == 0;
 }
 
 template <typename T>
@@ -1038,7 +1380,7 @@ namespace trtamd
 namespace
 {
 // Both entry points of the unfused attention after their own checks; inRegisters: the caller's one reading of
-// scores_in_registers for this call.
+// runs_in_one_launch for this call.
 int run_unfused(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d, void const* qkv,
     int32_t const* maskIdx, void* output, void* workspace, bool const inRegisters)
 {
@@ -1074,7 +1416,7 @@ extern "C" int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
         return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
     }
     return trtamd::run_unfused(stream, type, S, B, N, d, qkv, maskIdx, output, workspace,
-        trtamd::scores_in_registers(S, d));
+        trtamd::runs_in_one_launch(S, d));
 }
 
 extern "C" size_t trtamd_unfused_mha_static_capacity(void)
@@ -1099,9 +1441,9 @@ extern "C" int trtamd_unfused_mha_static(trtamd_stream_t stream, int32_t type, i
     {
         return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
     }
-    // Shapes of the one-launch kernel keep their scores in registers and touch nothing of the array: no limit for
-    // them.  Otherwise 2 * wordSize * S*S * B*N bytes, in double arithmetic free of overflow (each factor is below 2^31).
-    bool const inRegisters = trtamd::scores_in_registers(S, d);
+    // Shapes of the one-launch kernels (head sizes up to 128) keep their scores in registers and touch nothing of the
+    // array: no limit for them.  Otherwise 2 * wordSize * S*S * B*N bytes, in double arithmetic free of overflow (each factor is below 2^31).
+    bool const inRegisters = trtamd::runs_in_one_launch(S, d);
     double const need = 2.0 * (type == 0 ? 4.0 : 2.0) * (double) S * (double) S * (double) B * (double) N;
     if (!inRegisters && need > (double) kStaticScratchBytes)
     {

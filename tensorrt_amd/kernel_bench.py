@@ -315,8 +315,8 @@ def config_rows(api, torch, steps: int = 100, seed: int = 1, cpu: bool = True, l
                note="every query row of the S x B tensor is computed; ops count valid lengths only")
 
     # ---- unfused attention (FP32, other head sizes, S > 512) ------------------------------------------
-    # up to S = 512 and head size 128 one launch with a query's scores in registers; beyond, two MFMA GEMMs around
-    # a softmax with the S x S scores in the workspace
+    # head sizes up to 128: one launch, a query's scores in registers up to S = 512 and two passes over the keys beyond
+    # (larger head sizes: two MFMA GEMMs around a softmax with the S x S scores in the workspace)
     for dt, tname, type_id, peak in ((np.float16, "fp16", 1, PEAK_F16), (np.float32, "fp32", 0, PEAK_F32_MFMA)):
         for S, B, N, d in ((128, 32, 12, 64), (384, 32, 12, 64), (1024, 4, 12, 64)):
             hq = (r.standard_normal((S, B, 3 * N * d)) / 8).astype(dt)
@@ -328,9 +328,9 @@ def config_rows(api, torch, steps: int = 100, seed: int = 1, cpu: bool = True, l
             one = S <= 512
             report("C3 shape, unfused path",
                    "QKV-to-context v4 (attention_in_registers_kernel)" if one
-                   else "QKV-to-context v4 (batched_gemm_kernel x2 + softmax_rows_kernel)", tname,
+                   else "QKV-to-context v4 (attention_two_pass_kernel)", tname,
                    f"S={S} B={B} N={N} d={d}, all keys", t, ops=4.0 * d * N * B * S * S, peak_ops=peak,
-                   note="one launch, scores in registers" if one else "three launches, S x S scores through memory")
+                   note="one launch, scores in registers" if one else "one launch, two passes over the keys")
 
     # ---- C4: BERT-large INT8 layer, B=64, lengths U[192,384] -----------------------------------------
     wl = workloads.int8_layer(64, 384, N=16, seed=seed)

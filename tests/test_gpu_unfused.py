@@ -1,6 +1,6 @@
-"""GPU parity of the unfused attention path (the one-launch kernel that keeps a query's scores in registers for
-S <= 512 and head sizes <= 128, and the strided batched GEMMs around the scaled/masked softmax beyond that) and of
-zeroPadding2d, through the C ABI."""
+"""GPU parity of the unfused attention path (head sizes <= 128: one launch that keeps a query's scores in registers
+for S <= 512 and walks the keys twice beyond; larger head sizes: the strided batched GEMMs around the scaled/masked
+softmax) and of zeroPadding2d, through the C ABI."""
 import numpy as np
 import pytest
 
@@ -44,7 +44,11 @@ def test_scaled_softmax(api, dt, S, masked):
                                             (384, 1, 2, 64, True), (5, 2, 1, 8, False), (130, 2, 2, 128, True),
                                             # the last sizes of the one-launch kernel and the first beyond them
                                             (512, 1, 2, 64, True), (513, 1, 2, 64, True), (60, 2, 2, 129, True),
-                                            (250, 2, 3, 20, True), (1, 3, 2, 64, False), (65, 1, 1, 100, True)])
+                                            (250, 2, 3, 20, True), (1, 3, 2, 64, False), (65, 1, 1, 100, True),
+                                            # two passes over the keys: ragged last stage, every stage whole, head sizes
+                                            # that are not multiples of the vector width, no mask
+                                            (1024, 1, 2, 64, True), (1024, 2, 1, 64, False), (700, 2, 2, 72, True),
+                                            (1500, 1, 1, 128, True), (600, 1, 2, 33, True)])
 def test_unfused_mha(api, dt, S, B, N, d, masked):
     r = rng(210 + S + d)
     qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
@@ -81,7 +85,8 @@ def _run_unfused(api, dt, S, B, N, d, qkv, lens):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
-@pytest.mark.parametrize("S,B,N,d", [(384, 3, 4, 64), (200, 2, 2, 128), (97, 2, 3, 40), (512, 1, 2, 32)])
+@pytest.mark.parametrize("S,B,N,d", [(384, 3, 4, 64), (200, 2, 2, 128), (97, 2, 3, 40), (512, 1, 2, 32),
+                                     (640, 2, 2, 64), (1000, 1, 2, 128), (777, 2, 1, 40), (513, 1, 1, 8)])
 def test_one_launch_against_the_three_kernels(api, dt, S, B, N, d):
     """Both routes round scores and probabilities to the storage type at the same places; what is left between them
     is the order of the binary32 sums."""
