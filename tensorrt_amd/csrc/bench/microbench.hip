@@ -311,8 +311,9 @@ __global__ __launch_bounds__(512) void mfma_valu_split_kernel(int32_t const* src
                 for (int m = 0; m < 4; ++m)
                 {
                     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[m]) : "v"(a), "v"(b));
-                    // PAD x 8 idle cycles of this wavefront behind every MFMA (scalar no-ops, which do not use the
-                    // vector issue port): its next MFMA then arrives when the matrix pipe is free again
+                    // PAD scalar no-ops (`s_nop 7`, ~13 ns each as measured; they do not use the vector issue port)
+                    // behind every MFMA: with two or more, this wavefront's next MFMA arrives when the matrix pipe is
+                    // free again
 #pragma unroll
                     for (int p = 0; p < PAD; ++p)
                     {
@@ -468,7 +469,7 @@ MB_API float trtamd_microbench_valu(int op, int blocks, int iters, int32_t const
 
 // Milliseconds per launch of `blocks` workgroups of eight wavefronts: four that issue 4 * iters MFMAs each and four
 // that issue nv * iters v_fma_f32 each (nv 32 or 64); roles 1, 2 or 3 as described at the kernel; pad = number of
-// 8-cycle scalar no-ops behind every MFMA (0 .. 4).
+// `s_nop 7` behind every MFMA (0 .. 4).
 MB_API float trtamd_microbench_mfma_valu_split(int blocks, int iters, int nv, int pad, int roles, int32_t const* operands,
     int32_t* out)
 {

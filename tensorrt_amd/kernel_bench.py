@@ -118,7 +118,7 @@ def microbench(torch, cus: int = 256) -> dict:
                     ms = lib.trtamd_microbench_mfma_valu_split(cus * wgs, iters, nv, pad, roles, rnd.data_ptr(),
                                                                out.data_ptr())
                     t.append(round(ms * 1e-3 / iters * 1e9, 1))
-                split[f"wgs_per_cu={wgs},nv={nv},idle_cycles_behind_each_mfma={8 * pad}"] = t
+                split[f"wgs_per_cu={wgs},nv={nv},s_nop7_behind_each_mfma={pad}"] = t
     res["ns_per_iteration_[mfma_wavefronts_only,vector_wavefronts_only,both]_on_one_simd"] = split
     res["empty_launch_us"] = {f"{b}x{t}": round(lib.trtamd_microbench_empty(b, t, out.data_ptr()) * 1e3, 2)
                               for b, t in ((256, 256), (1041, 512), (2048, 256))}
