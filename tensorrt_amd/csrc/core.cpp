@@ -21,6 +21,7 @@ struct TuningEntry
 };
 constexpr TuningEntry kTuning[(int) Tuning::kCount] = {
     {"TRTAMD_LINEAR_PARTIAL_ROUND", 50}, {"TRTAMD_LINEAR_PERSISTENT", 1}, {"TRTAMD_LINEAR_DIRECT", 1},
+    {"TRTAMD_LINEAR_PIECES", 50},
     {"TRTAMD_FMHA_GENERIC", 0}, {"TRTAMD_FMHA_QSPLIT", 0}, {"TRTAMD_FMHA_RANKED", -1}, {"TRTAMD_UNFUSED_SPLIT", 0},
 };
 constexpr int kUnset = INT32_MIN;

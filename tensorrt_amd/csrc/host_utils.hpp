@@ -45,6 +45,7 @@ enum class Tuning : int
     kLinearPartialRound = 0, // TRTAMD_LINEAR_PARTIAL_ROUND=<percent>, default 50
     kLinearPersistent,       // TRTAMD_LINEAR_PERSISTENT=0/1, default 1
     kLinearDirect,           // TRTAMD_LINEAR_DIRECT=0/1, default 1
+    kLinearPieces,           // TRTAMD_LINEAR_PIECES=<percent>, default 50
     kFmhaGeneric,            // TRTAMD_FMHA_GENERIC=0/1, default 0
     kFmhaQsplit,             // TRTAMD_FMHA_QSPLIT=<n>, default 0 (chosen from the launch size)
     kFmhaRanked,             // TRTAMD_FMHA_RANKED=0/1, default -1 (chosen from the launch size)

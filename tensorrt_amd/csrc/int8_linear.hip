@@ -77,6 +77,7 @@ struct LinearArgs
     int tokMain;   // rows of 256 tokens they cover
     int panel;     // channel tiles per panel of the tile numbering (divides the number of channel tiles)
     int persist;   // persistent kernel: workgroups that loop over the 256 x 256 tiles
+    int pieces;    // direct-to-LDS kernel: the tokens behind the large tiles go in 64 x 64 pieces (see linear_piece64)
 };
 
 // gelu(y) = y * Phi(y) = max(y, 0) - |y| * Phi(-|y|).  log2(Phi(-a)) is smooth and nearly quadratic, so
@@ -987,6 +988,126 @@ __global__ __launch_bounds__(512) void int8_linear_persistent_kernel(LinearArgs 
     }
 }
 
+// A 64-channel x 64-token piece of the output for the tokens behind the large tiles, interleaved INT8 operands,
+// when those tokens would make only a few 128 x 128 tiles (a long k loop on a few CUs while the others idle).
+// The eight wavefronts split k, not the piece: wavefront w multiplies the k-slabs w, w + 8, ... of all four 32 x 32
+// blocks.  In the interleaved layout a fragment (32 rows x 32 bytes of one k-slab) is 1 KB of consecutive memory in
+// exactly the order the MFMA wants it from the lanes, so every fragment is one 16-byte load per lane straight into the
+// operand registers: no LDS stage, no barrier in the loop, and no byte is fetched twice by the workgroup.  The eight
+// partial accumulators meet in LDS (8 x 16 KB), four wavefronts add them up, one block each, and run the epilogue.
+// Integer addition is exact, so the result is the bits of any other order.  K % 256 == 0, N % 64 == 0.
+template <bool IL_OUT, int EPI>
+__device__ __forceinline__ void linear_piece64(
+    LinearArgs const& p, int const n0, int const t0, uint8_t* __restrict__ lds, float* sScale)
+{
+    static_assert(EPI == kAFFINE || EPI == kGELU, "INT8 outputs");
+    constexpr int kDepth = 4; // k-slabs in flight per wavefront
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const row = lane & 31, half = lane >> 5;
+    // channel and token rows of this lane in the two row blocks of each operand; tokens beyond T re-read the last one
+    uint32_t offA[2], offB[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+    {
+        offA[b] = (uint32_t) (n0 + 32 * b + row) * 32u + (uint32_t) half * 16u;
+        offB[b] = (uint32_t) min(t0 + 32 * b + row, p.T - 1) * 32u + (uint32_t) half * 16u;
+    }
+    uint32_t const slabA = (uint32_t) p.N * 32u, slabB = (uint32_t) p.T * 32u;
+    int const steps = p.K / 256; // k-slabs of this wavefront
+    if (threadIdx.x < 64)
+    {
+        sScale[threadIdx.x] = p.alpha[n0 + threadIdx.x];
+        sScale[kBigTile + threadIdx.x] = p.beta[n0 + threadIdx.x];
+    }
+    i32x4 fa[kDepth][2], fb[kDepth][2];
+    auto fetch = [&](int slot, int step) {
+        uint32_t const ks = (uint32_t) (min(step, steps - 1) * 8 + wave);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+        {
+            fa[slot][b] = *reinterpret_cast<i32x4 const*>(p.w + (size_t) ks * slabA + offA[b]);
+            fb[slot][b] = *reinterpret_cast<i32x4 const*>(p.a + (size_t) ks * slabB + offB[b]);
+        }
+    };
+    AccT<EPI> acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+    {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+        {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+            {
+                acc[i][j][v] = 0;
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+    {
+        fetch(d, d);
+    }
+    for (int s0 = 0; s0 < steps; s0 += kDepth)
+    {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d)
+        {
+            if (s0 + d < steps)
+            {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                    {
+                        acc[i][j] = mma<EPI>(fa[d][i], fb[d][j], acc[i][j]);
+                    }
+                }
+                fetch(d, s0 + d + kDepth); // loads behind the last slab re-read it and are never used
+            }
+        }
+    }
+    // partial accumulators: [wavefront][block][four registers][lane], 16 bytes per lane and access
+    i32x4* const part = reinterpret_cast<i32x4*>(lds);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+    {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+        {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                part[(((wave * 4) + (i * 2 + j)) * 4 + q) * 64 + lane]
+                    = i32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            }
+        }
+    }
+    __syncthreads();
+    if (wave < 4)
+    {
+        AccT<EPI> sum;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            i32x4 t = part[((wave) * 4 + q) * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < 8; ++w)
+            {
+                t += part[(((w * 4) + wave) * 4 + q) * 64 + lane];
+            }
+            sum[4 * q] = t[0];
+            sum[4 * q + 1] = t[1];
+            sum[4 * q + 2] = t[2];
+            sum[4 * q + 3] = t[3];
+        }
+        int const cb = (wave >> 1) * 32, tb = (wave & 1) * 32;
+        store_block<IL_OUT, EPI>(p, sum, n0 + cb, t0 + tb, sScale + cb, sScale + kBigTile + cb);
+    }
+}
+
 // The persistent tile plan with direct-to-LDS loads for the 256 x 256 tiles.
 template <bool IL, bool IL_OUT, int EPI>
 __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p)
@@ -1008,8 +1129,18 @@ __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p
     }
     else
     {
-        uint32_t const nbm = (uint32_t) ((p.N + kSmall - 1) / kSmall);
         uint32_t const tile = blockIdx.x - (uint32_t) p.persist;
+        if constexpr (IL && (EPI == kAFFINE || EPI == kGELU))
+        {
+            if (p.pieces)
+            {
+                uint32_t const nbm = (uint32_t) p.N / 64u;
+                linear_piece64<IL_OUT, EPI>(p, (int) (tile % nbm) * 64, p.tokMain * kBig + (int) (tile / nbm) * 64, lds,
+                    sScale);
+                return;
+            }
+        }
+        uint32_t const nbm = (uint32_t) ((p.N + kSmall - 1) / kSmall);
         auto origin = [&](int, int& n0, int& t0) {
             n0 = (int) (tile % nbm) * kSmall;
             t0 = p.tokMain * kBig + (int) (tile / nbm) * kSmall;
@@ -1074,7 +1205,20 @@ int launch_shape(hipStream_t stream, LinearArgs a)
         {
             if (direct && a.N % kBig == 0 && a.K % 256 == 0 && a.mainTiles > 0)
             {
-                hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI>), dim3((uint32_t) pgrid), dim3(512), 0, stream,
+                int64_t dgrid = pgrid;
+                if constexpr (IL_W && (EPI == kAFFINE || EPI == kGELU))
+                {
+                    // few 128 x 128 tiles behind the large ones (no more than TRTAMD_LINEAR_PIECES per cent of the CUs
+                    // busy with a long k loop each): the same tokens as 64 x 64 pieces whose wavefronts split k
+                    // (linear_piece64)
+                    int64_t const smallTiles = grid - a.mainTiles;
+                    if (restTokens > 0 && smallTiles * 100 <= (int64_t) tuning(Tuning::kLinearPieces) * cus)
+                    {
+                        a.pieces = 1;
+                        dgrid = (int64_t) a.persist + (int64_t) (a.N / 64) * ceil_div(restTokens, 64);
+                    }
+                }
+                hipLaunchKernelGGL((int8_linear_dma_kernel<IL_W, IL_OUT, EPI>), dim3((uint32_t) dgrid), dim3(512), 0, stream,
                     a);
                 return check_launch("int8_linear_dma_kernel");
             }

@@ -38,6 +38,28 @@ LINEAR_SETTINGS = [("TRTAMD_LINEAR_DIRECT", 0), ("TRTAMD_LINEAR_PERSISTENT", 0),
                    ("TRTAMD_LINEAR_PARTIAL_ROUND", 100)]
 
 
+def test_remainder_pieces_against_remainder_tiles():
+    """More than half a round of large tiles (so that they run, as a partial round) and 60 tokens behind them: by
+    default those go in 64 x 64 pieces whose wavefronts split k, with TRTAMD_LINEAR_PIECES=0 in 128 x 128 tiles; both
+    must give the oracle's accumulator-exact results and the same bytes."""
+    T, K, N = 133 * 256 + 60, 256, 512
+    a, w, alpha, beta = problem(93, T, K, N)
+    ref = oracle.int8_linear(a, w, alpha, beta, oracle.LINEAR_AFFINE, out_interleaved=True)
+    pieces = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=True, out_il=True, w_il=True)
+    with tuning("TRTAMD_LINEAR_PIECES", 0):
+        tiles = run_gpu(a, w, alpha, beta, capi.LINEAR_AFFINE, a_il=True, out_il=True, w_il=True)
+    assert_int8_close(pieces, ref, what="pieces", max_frac_off=1e-3)
+    assert np.array_equal(pieces, tiles)
+    q = float(np.float32(127.0 / 4.0))
+    al, be = (alpha * 0.06).astype(np.float32), (beta * 0.02).astype(np.float32)
+    ref = oracle.int8_linear(a, w, al, be, oracle.LINEAR_GELU, out_scale=q, out_interleaved=True)
+    pieces = run_gpu(a, w, al, be, capi.LINEAR_GELU, out_scale=q, a_il=True, out_il=True, w_il=True)
+    with tuning("TRTAMD_LINEAR_PIECES", 0):
+        tiles = run_gpu(a, w, al, be, capi.LINEAR_GELU, out_scale=q, a_il=True, out_il=True, w_il=True)
+    assert_int8_close(pieces, ref, what="pieces, GELU", max_frac_off=2e-3)
+    assert np.array_equal(pieces, tiles)
+
+
 @pytest.mark.parametrize("name,value", LINEAR_SETTINGS)
 @pytest.mark.parametrize("il", [True, False])
 def test_linear_variants(name, value, il):
