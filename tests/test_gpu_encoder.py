@@ -64,6 +64,42 @@ def test_embedding_and_quantiser(setup):
 
 @pytest.mark.parametrize("layer", [0, 1])
 def test_layer_operations(setup, layer):
+    check_layer(setup, layer)
+
+
+@pytest.fixture(scope="module")
+def setup_large():
+    """The benchmark's network (BERT-large: hidden 1024, 16 heads, feed-forward 4096, 24 layers) on a few short
+    sequences, so that the oracle can follow every operation of every layer in seconds."""
+    cfg = EncoderConfig(hidden=1024, heads=16, ffn=4096, layers=24, vocab=1000, max_pos=512, max_seqlen=384, seed=11)
+    enc = Int8BertEncoder(cfg)
+    r = rng(12)
+    lens = np.array([33, 384, 1, 140])
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    ids = r.integers(0, cfg.vocab, T).astype(np.int32)
+    segs = r.integers(0, 2, T).astype(np.int32)
+    enc.calibrate(ids, segs, cu)
+    cap = {}
+    out = enc.enqueue(ids, segs, cu, capture=cap)
+    import torch
+    torch.cuda.synchronize()
+    return cfg, enc, ids, segs, cu, cap, out.cpu().numpy()
+
+
+def test_every_layer_of_the_24_layer_network(setup_large):
+    """Depth: the same per-operation checks on all 24 layers of the benchmark's network, each operation against the
+    oracle applied to the tensor the GPU chain fed it, down to the dequantised output."""
+    cfg, enc, ids, segs, cu, cap, out = setup_large
+    for layer in range(cfg.layers):
+        check_layer(setup_large, layer)
+    want = oracle.dequantize_deinterleave_f16(cap["x_out"], enc.layers[-1]["scales"]["out"])
+    assert np.array_equal(out, want)
+    # the chain has not collapsed on the way down: the last layer still uses the INT8 range
+    assert int(np.abs(cap["x_out"].astype(np.int32)).max()) >= 100
+
+
+def check_layer(setup, layer):
     cfg, enc, ids, segs, cu, cap, _ = setup
     T, E, F, N = int(cu[-1]), cfg.hidden, cfg.ffn, cfg.heads
     L, sc = enc.layers[layer], enc.layers[layer]["scales"]
