@@ -155,6 +155,28 @@ TRTAMD_API size_t trtamd_unfused_mha_workspace_size(int32_t type, int32_t S, int
 TRTAMD_API int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t S, int32_t B, int32_t N, int32_t d,
     void const* qkv, int32_t const* maskIdx, void* output, void* workspace);
 
+/* The algorithm choice of the unfused runner.  The reference times cuBLAS's batched-GEMM algorithms for the configured
+ * shape once, when the runner is set up, keeps the two winners (mAlgoBatchedEx1 / mAlgoBatchedEx2) in its serialised
+ * state and passes them to every later product (tuneBatchedGemm and UnfusedMHARunner::setup / serialize,
+ * plugin/bertQKVToContextPlugin/mhaRunner.cu:346-444, 476-507, 527-601).  Here what there is to choose for a shape is
+ * the route: one launch that stores no score, or the three launches with the score matrices in the workspace.
+ * trtamd_unfused_mha_tune times the routes that exist for the shape on buffers of its own (allocated and freed inside
+ * the call: it is for configuration time, not for enqueue; the batch is cut down for the timing when the workspace
+ * would exceed 1 GiB) and returns the faster one in *route and, when `microseconds` is not NULL, the two times
+ * (microseconds[0] one launch, [1] three launches; -1 for a route that does not exist or was not timed).  When nothing
+ * can be timed (no device memory for the buffers) it returns TRTAMD_UNFUSED_ROUTE_BY_SHAPE, which is also the
+ * reference's default algorithm value, so that a state that was never tuned, or was written by the reference, reads as
+ * "choose by shape".  trtamd_unfused_mha_routed is trtamd_unfused_mha with the route given: BY_SHAPE behaves as
+ * trtamd_unfused_mha does, ONE_LAUNCH is refused for head sizes above 128, any other value is a bad parameter.
+ * The routes round at the same places and differ in the order of binary32 sums only. */
+#define TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH 0
+#define TRTAMD_UNFUSED_ROUTE_THREE_LAUNCHES 1
+#define TRTAMD_UNFUSED_ROUTE_BY_SHAPE 99
+TRTAMD_API int trtamd_unfused_mha_tune(int32_t type, int32_t S, int32_t B, int32_t N, int32_t d, int32_t* route,
+    float* microseconds);
+TRTAMD_API int trtamd_unfused_mha_routed(trtamd_stream_t stream, int32_t route, int32_t type, int32_t S, int32_t B,
+    int32_t N, int32_t d, void const* qkv, int32_t const* maskIdx, void* output, void* workspace);
+
 /* trtamd_unfused_mha for callers that cannot allocate (code under graph capture, tight serving loops, harnesses
  * that forbid hipMalloc).  No counterpart in the reference: the score matrices live in a device array that belongs to
  * the library (trtamd_unfused_mha_static_capacity() bytes, 32 MiB, held by every GPU the library runs on until the

@@ -50,6 +50,7 @@ class Fp16LinearParams(C.Structure):
 
 
 LINEAR_AFFINE, LINEAR_GELU, LINEAR_RAW_INT32, LINEAR_AFFINE_FP16 = 0, 1, 2, 3
+UNFUSED_ROUTE_ONE_LAUNCH, UNFUSED_ROUTE_THREE_LAUNCHES, UNFUSED_ROUTE_BY_SHAPE = 0, 1, 99
 
 
 class EncoderConfig(C.Structure):
@@ -106,6 +107,8 @@ _SIGS = {
     "trtamd_scaled_softmax_fp16": (C.c_int, [c_p, i32, i32, i32, f32, c_p, c_p, c_p]),
     "trtamd_unfused_mha_workspace_size": (C.c_size_t, [i32, i32, i32, i32]),
     "trtamd_unfused_mha": (C.c_int, [c_p, i32, i32, i32, i32, i32, c_p, c_p, c_p, c_p]),
+    "trtamd_unfused_mha_routed": (C.c_int, [c_p, i32, i32, i32, i32, i32, i32, c_p, c_p, c_p, c_p]),
+    "trtamd_unfused_mha_tune": (C.c_int, [i32, i32, i32, i32, i32, C.POINTER(C.c_int32), C.POINTER(C.c_float)]),
     "trtamd_unfused_mha_static_capacity": (C.c_size_t, []),
     "trtamd_unfused_mha_static_prepare": (C.c_int, []),
     "trtamd_test_set_tuning": (C.c_int, [C.c_char_p, i32]),

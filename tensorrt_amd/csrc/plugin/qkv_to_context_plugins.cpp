@@ -21,7 +21,8 @@ namespace
 constexpr char const* kNAME = "CustomQKVToContextPluginDynamic";
 constexpr int32_t kIIDX = 0; // packed QKV
 constexpr int32_t kMIDX = 1; // mask
-constexpr int32_t kDefaultGemmAlgo = 99; // CUBLAS_GEMM_DEFAULT_TENSOR_OP: kept so serialised state has the reference's layout
+// CUBLAS_GEMM_DEFAULT_TENSOR_OP, the value the reference's runner holds before it has tuned; here "route by shape"
+constexpr int32_t kDefaultGemmAlgo = TRTAMD_UNFUSED_ROUTE_BY_SHAPE;
 
 uint32_t floatBits(float f)
 {
@@ -39,12 +40,47 @@ uint32_t half2Bits(float f)
 // Geometry of MHARunner::setup (plugin/bertQKVToContextPlugin/mhaRunner.h:62-83) plus which
 // runner it belongs to; (de)serialised in the reference's byte layout
 // (mhaRunner.cu:456-474 for the fused runners, :489-507 for the unfused one).
+// The unfused runner's first algorithm slot holds the route that trtamd_unfused_mha_tune found fastest for the configured
+// shape (the reference keeps the cuBLAS algorithms of its two batched products there, found the same way at set-up:
+// mhaRunner.cu:346-444, 476-487); the second slot has nothing to hold and stays at the default.
 struct RunnerState
 {
     bool unfused{false};
     bool setUp{false};
     int32_t S{0}, B{0}, headSize{0};
     int32_t algo1{kDefaultGemmAlgo}, algo2{kDefaultGemmAlgo};
+    int32_t tunedS{0}, tunedB{0}; // the shape algo1 was timed for (0: never)
+
+    // UnfusedMHARunner::setup's "if (!mIsBestAlgoFound)" step: once per configured shape, at build time, on the
+    // device of the calling thread; without a device (or when the timing fails) the route stays with the shape
+    void tune(DataType type, int32_t numHeads)
+    {
+        if (!unfused || !setUp || (tunedS == S && tunedB == B) || type == DataType::kINT8 || !deviceAvailable())
+        {
+            return;
+        }
+        int32_t route = kDefaultGemmAlgo;
+        if (trtamd_unfused_mha_tune(static_cast<int32_t>(type), S, B, numHeads, headSize, &route, nullptr)
+            == TRTAMD_STATUS_SUCCESS)
+        {
+            algo1 = route;
+        }
+        else
+        {
+            logMessage(ILogger::Severity::kWARNING,
+                std::string("the unfused attention routes could not be timed: ") + trtamd_last_error());
+            algo1 = kDefaultGemmAlgo;
+        }
+        tunedS = S;
+        tunedB = B;
+    }
+    // what enqueue passes on: a route this library knows, or "by shape" for anything else a stream may hold (the
+    // reference writes cuBLAS algorithm numbers there)
+    int32_t route() const
+    {
+        bool const oneLaunch = algo1 == TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH && headSize <= 128;
+        return oneLaunch || algo1 == TRTAMD_UNFUSED_ROUTE_THREE_LAUNCHES ? algo1 : TRTAMD_UNFUSED_ROUTE_BY_SHAPE;
+    }
 
     void setup(int32_t s, int32_t b, int32_t d)
     {
@@ -155,8 +191,8 @@ int32_t runUnfused(DataType type, RunnerState const& st, int32_t numHeads, void 
 {
     TRTAMD_VALIDATE_MSG(type != DataType::kINT8, "The Unfused MHARunner does not support INT8!");
     TRTAMD_VALIDATE(workspace != nullptr);
-    checkKernelStatus(trtamd_unfused_mha(stream, static_cast<int32_t>(type), st.S, st.B, numHeads, st.headSize, qkv,
-                          static_cast<int32_t const*>(maskIdx), output, workspace),
+    checkKernelStatus(trtamd_unfused_mha_routed(stream, st.route(), static_cast<int32_t>(type), st.S, st.B, numHeads,
+                          st.headSize, qkv, static_cast<int32_t const*>(maskIdx), output, workspace),
         "unfused attention");
     return 0;
 }
@@ -333,6 +369,7 @@ protected:
             mS = S;
             mB = B;
         }
+        mUnfused.tune(mType, mNumHeads);
     }
 
     size_t doWorkspaceSize(DynamicPluginTensorDesc const*, DynamicPluginTensorDesc const*) const override
@@ -710,6 +747,7 @@ protected:
                 mS = S;
                 mB = B;
             }
+            mRunner.tune(mType, mNumHeads);
         }
         else
         {

@@ -498,7 +498,6 @@ int can_vectorise(T const* base, GemmOperand const& o)
 // ------------------------------------------------------------------------------------------
 constexpr int kRegQueries = 64; // queries per workgroup
 constexpr int kRegKeys = 64;    // keys per LDS stage
-constexpr int kRegMaxS = 512;  // keys whose scores one lane can hold (32 tiles); longer sequences walk the keys twice
 constexpr int kRegMaxD = 128;
 
 template <typename T, int DP>
@@ -1417,6 +1416,134 @@ extern "C" int trtamd_unfused_mha(trtamd_stream_t stream, int32_t type, int32_t 
     }
     return trtamd::run_unfused(stream, type, S, B, N, d, qkv, maskIdx, output, workspace,
         trtamd::runs_in_one_launch(S, d));
+}
+
+extern "C" int trtamd_unfused_mha_routed(trtamd_stream_t stream, int32_t route, int32_t type, int32_t S, int32_t B,
+    int32_t N, int32_t d, void const* qkv, int32_t const* maskIdx, void* output, void* workspace)
+{
+    if (route == TRTAMD_UNFUSED_ROUTE_BY_SHAPE)
+    {
+        return trtamd_unfused_mha(stream, type, S, B, N, d, qkv, maskIdx, output, workspace);
+    }
+    if (route != TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH && route != TRTAMD_UNFUSED_ROUTE_THREE_LAUNCHES)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: unknown route %d", route);
+    }
+    if (type != 0 && type != 1)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: data type %d (only FP32=0 and FP16=1)", type);
+    }
+    if (S <= 0 || B <= 0 || N <= 0 || d <= 0)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
+    }
+    if (route == TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH && d > trtamd::kRegMaxD)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: no one-launch kernel for head size %d (limit %d)", d,
+            trtamd::kRegMaxD);
+    }
+    return trtamd::run_unfused(stream, type, S, B, N, d, qkv, maskIdx, output, workspace,
+        route == TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH);
+}
+
+extern "C" int trtamd_unfused_mha_tune(
+    int32_t type, int32_t S, int32_t B, int32_t N, int32_t d, int32_t* route, float* microseconds)
+{
+    using namespace trtamd;
+    if (route == nullptr)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA tuning: null route pointer");
+    }
+    *route = TRTAMD_UNFUSED_ROUTE_BY_SHAPE;
+    float us[2] = {-1.f, -1.f};
+    auto report = [&] {
+        if (microseconds)
+        {
+            microseconds[0] = us[0];
+            microseconds[1] = us[1];
+        }
+    };
+    report();
+    if (type != 0 && type != 1)
+    {
+        return set_error(TRTAMD_STATUS_NOT_SUPPORTED, "unfused MHA: data type %d (only FP32=0 and FP16=1)", type);
+    }
+    if (S <= 0 || B <= 0 || N <= 0 || d <= 0 || (int64_t) B * N > 65535)
+    {
+        return set_error(TRTAMD_STATUS_BAD_PARAM, "unfused MHA: bad dimensions S=%d B=%d N=%d d=%d", S, B, N, d);
+    }
+    if (d > kRegMaxD)
+    {
+        *route = TRTAMD_UNFUSED_ROUTE_THREE_LAUNCHES; // the only route there is
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    // the timed problem: the configured one, with the batch halved until the score matrices fit 1 GiB
+    constexpr size_t kMaxWorkspace = (size_t) 1 << 30;
+    int32_t bt = B;
+    while (bt > 1 && trtamd_unfused_mha_workspace_size(type, S, bt, N) > kMaxWorkspace)
+    {
+        bt = (bt + 1) / 2;
+    }
+    size_t const wsBytes = trtamd_unfused_mha_workspace_size(type, S, bt, N);
+    if (wsBytes > kMaxWorkspace)
+    {
+        return TRTAMD_STATUS_SUCCESS; // by shape
+    }
+    size_t const word = type == 0 ? 4 : 2;
+    size_t const outBytes = word * (size_t) S * (size_t) bt * (size_t) N * (size_t) d;
+    void *qkv = nullptr, *out = nullptr, *ws = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto release = [&] {
+        if (e0) (void) hipEventDestroy(e0);
+        if (e1) (void) hipEventDestroy(e1);
+        if (stream) (void) hipStreamDestroy(stream);
+        if (qkv) (void) hipFree(qkv);
+        if (out) (void) hipFree(out);
+        if (ws) (void) hipFree(ws);
+    };
+    bool ok = hipMalloc(&qkv, 3 * outBytes) == hipSuccess && hipMalloc(&out, outBytes) == hipSuccess
+        && hipMalloc(&ws, wsBytes) == hipSuccess && hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) == hipSuccess
+        && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
+    // every element the same small positive number (0x3c3c... is 1.06 in binary16 and 0.0115 in binary32)
+    ok = ok && hipMemsetAsync(qkv, 0x3c, 3 * outBytes, stream) == hipSuccess;
+    if (!ok)
+    {
+        (void) hipGetLastError(); // best effort: without buffers the choice stays with the shape
+        release();
+        return TRTAMD_STATUS_SUCCESS;
+    }
+    constexpr int kWarm = 2, kTimed = 5;
+    int status = TRTAMD_STATUS_SUCCESS;
+    for (int r = 0; r < 2 && status == TRTAMD_STATUS_SUCCESS; ++r)
+    {
+        for (int i = 0; i < kWarm + kTimed && status == TRTAMD_STATUS_SUCCESS; ++i)
+        {
+            if (i == kWarm && hipEventRecord(e0, stream) != hipSuccess)
+            {
+                status = set_error(TRTAMD_STATUS_FAILURE, "unfused MHA tuning: event record failed");
+                break;
+            }
+            status = run_unfused(stream, type, S, bt, N, d, qkv, nullptr, out, ws, r == TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH);
+        }
+        float ms = 0.f;
+        if (status == TRTAMD_STATUS_SUCCESS
+            && (hipEventRecord(e1, stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess
+                || hipEventElapsedTime(&ms, e0, e1) != hipSuccess))
+        {
+            status = set_error(TRTAMD_STATUS_FAILURE, "unfused MHA tuning: timing failed");
+        }
+        us[r] = ms * 1000.f / kTimed;
+    }
+    (void) hipStreamSynchronize(stream);
+    release();
+    if (status != TRTAMD_STATUS_SUCCESS)
+    {
+        return status;
+    }
+    *route = us[1] < us[0] ? TRTAMD_UNFUSED_ROUTE_THREE_LAUNCHES : TRTAMD_UNFUSED_ROUTE_ONE_LAUNCH;
+    report();
+    return TRTAMD_STATUS_SUCCESS;
 }
 
 extern "C" size_t trtamd_unfused_mha_static_capacity(void)

@@ -330,6 +330,43 @@ def test_qkv_unfused_path(reg, version, dt, S, has_mask):
     assert_fp_close(host(out), ref, what="unfused attention")
 
 
+@pytest.mark.parametrize("version", ["4", "5"])
+def test_qkv_unfused_route_is_tuned_at_configure_and_travels_with_the_state(reg, version):
+    """configurePlugin on a GPU times the unfused routes for the shape and writes the faster one into the first
+    algorithm slot of the serialised runner state; a runtime plugin follows whatever the slot holds (either route, the
+    default, a cuBLAS algorithm number written by the reference) to the same result."""
+    r = rng(150)
+    S, B, N, d = 70, 3, 2, 48
+    hidden = N * d
+    dt, npdt = DataType.HALF, np.float16
+    qkv = r.standard_normal((S, B, 3 * hidden)).astype(npdt)
+    lens = r.integers(1, S + 1, B).astype(np.int32)
+    c = reg.get_creator(QKV, version)
+    p = c.create_plugin("qkv", qkv_fields(int(dt), hidden, N, 1))
+    ins = [TensorDesc([S, B, 3 * hidden, 1, 1], dt),
+           TensorDesc([B, 1], DataType.INT32) if version == "4" else TensorDesc([B], DataType.INT32)]
+    outs = [TensorDesc([S, B, hidden, 1, 1], dt)]
+    assert p.configure_plugin(ins, outs) == 0, last_log()
+    fields = p.get_fields_to_serialize()
+    state = next(f for f in fields if f.name == "runnerStateBuffer")
+    words = state.data.view(np.int32)
+    assert words.tolist()[1:] == [99, S, B, d]
+    assert words[0] in (0, 1), "the route found at configure time"
+    ref = oracle.mha_unfused_fixed(qkv, S, B, N, d, lens)
+    ws = dev_empty((p.get_workspace_size(ins, outs),), np.uint8)
+    for slot in (0, 1, 99, 103):
+        forged = [f if f.name != "runnerStateBuffer" else
+                  PluginField("runnerStateBuffer", np.array([slot, 99, S, B, d], np.int32).view(np.uint8), f.type)
+                  for f in fields]
+        rt = c.create_plugin("rt", forged, TensorRTPhase.RUNTIME)
+        assert rt is not None, last_log()
+        out = dev_empty((S, B, hidden), npdt, fill=0)
+        run(rt, ins, outs, [dev(qkv), dev(lens)], [out], ws)
+        assert_fp_close(host(out), ref, what=f"unfused attention, slot {slot}")
+        kept = next(f for f in rt.get_fields_to_serialize() if f.name == "runnerStateBuffer").data.view(np.int32)
+        assert kept.tolist() == [slot, 99, S, B, d], "a runtime plugin keeps the state it was given"
+
+
 @pytest.mark.parametrize("dt,d", [(DataType.HALF, 64), (DataType.INT8, 64), (DataType.HALF, 32), (DataType.INT8, 32),
                                   (DataType.HALF, 40)])
 def test_qkv_v5_varseqlen(reg, dt, d):

@@ -1,11 +1,16 @@
 """GPU parity of the unfused attention path (head sizes <= 128: one launch that keeps a query's scores in registers
 for S <= 512 and walks the keys twice beyond; larger head sizes: the strided batched GEMMs around the scaled/masked
 softmax) and of zeroPadding2d, through the C ABI."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
 import oracle
 from helpers import assert_fp_close, attention_f64, dev, dev_empty, host, ptr, rng, stream, sync
+from tensorrt_amd import capi
+
+STATUS_BAD_PARAM, STATUS_NOT_SUPPORTED = 2, 3
 
 pytestmark = pytest.mark.gpu
 
@@ -104,6 +109,61 @@ def test_one_launch_against_the_three_kernels(api, dt, S, B, N, d):
     assert_fp_close(one, split, what="one launch vs three kernels", **tol)
     assert_fp_close(one, oracle.mha_unfused_fixed(qkv, S, B, N, d, lens), what="vs oracle",
                     **(dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}))
+
+
+def _run_routed(api, route, dt, S, B, N, d, qkv, lens):
+    ws = dev_empty((api.unfused_mha_workspace_size(0 if dt == np.float32 else 1, S, B, N),), np.uint8)
+    out = dev_empty((S, B, N * d), dt, fill=0)
+    d_qkv, d_len = dev(qkv), dev(lens)    # held until the result is back
+    st = api.unfused_mha_routed(stream(), route, 0 if dt == np.float32 else 1, S, B, N, d, ptr(d_qkv), ptr(d_len),
+                                ptr(out), ptr(ws))
+    sync()
+    return st, host(out)
+
+
+@pytest.mark.parametrize("dt,S,B,N,d", [(np.float16, 300, 3, 4, 64), (np.float32, 640, 2, 2, 128),
+                                        (np.float16, 1030, 2, 3, 80), (np.float32, 77, 5, 2, 24)])
+def test_routes_and_their_tuning(api, dt, S, B, N, d):
+    """The route can be named; both give the oracle's result, "by shape" is the default entry point, and the tuning
+    call times both and returns the faster."""
+    r = rng(870 + S)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(dt)
+    lens = r.integers(1, S + 1, B).astype(np.int32)
+    ref = oracle.mha_unfused_fixed(qkv, S, B, N, d, lens)
+    tol = dict(atol=2e-5, rtol=1e-4) if dt == np.float32 else {}
+    got = {}
+    for route in (capi.UNFUSED_ROUTE_ONE_LAUNCH, capi.UNFUSED_ROUTE_THREE_LAUNCHES, capi.UNFUSED_ROUTE_BY_SHAPE):
+        st, got[route] = _run_routed(api, route, dt, S, B, N, d, qkv, lens)
+        assert st == 0, api.last_error_str()
+        assert_fp_close(got[route], ref, what=f"route {route} vs oracle", **tol)
+    assert np.array_equal(got[capi.UNFUSED_ROUTE_BY_SHAPE], _run_unfused(api, dt, S, B, N, d, qkv, lens))
+    assert np.array_equal(got[capi.UNFUSED_ROUTE_BY_SHAPE], got[capi.UNFUSED_ROUTE_ONE_LAUNCH]), "head sizes <= 128"
+    route, us = C.c_int32(-5), (C.c_float * 2)(0, 0)
+    api.check(api.unfused_mha_tune(0 if dt == np.float32 else 1, S, B, N, d, C.byref(route), us))
+    assert us[0] > 0 and us[1] > 0
+    assert route.value == (capi.UNFUSED_ROUTE_THREE_LAUNCHES if us[1] < us[0] else capi.UNFUSED_ROUTE_ONE_LAUNCH)
+
+
+def test_routes_that_do_not_exist(api):
+    S, B, N, d = 40, 2, 2, 136
+    r = rng(880)
+    qkv = r.standard_normal((S, B, 3 * N * d)).astype(np.float16)
+    lens = np.array([40, 9], np.int32)
+    st, _ = _run_routed(api, capi.UNFUSED_ROUTE_ONE_LAUNCH, np.float16, S, B, N, d, qkv, lens)
+    assert st == STATUS_NOT_SUPPORTED and "head size" in api.last_error_str()
+    st, _ = _run_routed(api, 7, np.float16, S, B, N, d, qkv, lens)
+    assert st == STATUS_BAD_PARAM and "route" in api.last_error_str()
+    st, got = _run_routed(api, capi.UNFUSED_ROUTE_THREE_LAUNCHES, np.float16, S, B, N, d, qkv, lens)
+    assert st == 0
+    assert_fp_close(got, oracle.mha_unfused_fixed(qkv, S, B, N, d, lens), what="three launches, head size 136")
+    # above 128 there is one route and nothing to time
+    route, us = C.c_int32(-5), (C.c_float * 2)(0, 0)
+    api.check(api.unfused_mha_tune(1, S, B, N, d, C.byref(route), us))
+    assert route.value == capi.UNFUSED_ROUTE_THREE_LAUNCHES and us[0] == -1 and us[1] == -1
+    assert api.unfused_mha_tune(2, S, B, N, 64, C.byref(route), None) == STATUS_NOT_SUPPORTED
+    assert route.value == capi.UNFUSED_ROUTE_BY_SHAPE
+    assert api.unfused_mha_tune(1, 0, B, N, 64, C.byref(route), None) == STATUS_BAD_PARAM
+    assert api.unfused_mha_tune(1, S, B, N, 64, None, None) == STATUS_BAD_PARAM
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float16])
