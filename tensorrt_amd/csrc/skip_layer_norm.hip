@@ -411,6 +411,27 @@ __global__ __launch_bounds__(kBlock) void skipln_dqq_kernel(int const ld, int64_
 // in*skip, sum skip^2) combined in binary64, so mean and variance carry no accumulation error.
 // gamma*qScale and beta*qScale are staged once per workgroup in LDS as binary32.
 // ------------------------------------------------------------------------------------------
+// Which block of TOK consecutive tokens a workgroup takes.  Workgroup ids are dealt round-robin to the 8 XCDs, each
+// with an L2 of its own, and neighbouring token blocks touch the same cache lines at their common border in all 32
+// channel groups whenever a group's rows do not start on a line (32 bytes per token: any token count that is not a
+// multiple of 4): in id order both neighbours fetch those lines from memory and write them back in halves.  Runs of 64
+// consecutive blocks therefore go to one XCD (ids 512 m + 8 r + x -> block 512 m + 64 x + r), and what is left
+// behind the last whole span of 512 is dealt the same way in shorter runs.  Measured at 33289 tokens x 1024 channels:
+// 19.5 -> 17.8 us with the tensors in the last-level cache, unchanged from memory (longer runs, up to one run per
+// XCD, lose 3 % there); 65536 tokens, whose group stride is a power of two, 52.9 -> 31.5 us.
+__device__ inline uint32_t token_block_of_workgroup(uint32_t bid, uint32_t nblocks)
+{
+    constexpr uint32_t kXcds = 8, kRun = 64, kSpan = kXcds * kRun;
+    uint32_t const first = bid / kSpan * kSpan; // first id of this workgroup's span
+    uint32_t const x = bid - first;
+    uint32_t const run = first + kSpan <= nblocks ? kRun : (nblocks - first) / kXcds;
+    if (x >= run * kXcds)
+    {
+        return bid; // the last few ids of a short span keep their blocks
+    }
+    return first + (x % kXcds) * run + x / kXcds;
+}
+
 template <int G, int W, int TOK, bool PRELN>
 __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int const total,
     int8_t const* __restrict__ in, int8_t const* __restrict__ skip, f16 const* __restrict__ beta,
@@ -435,7 +456,7 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
     int const sub = lane / LPG;
     int const tok = (lane % LPG) >> 1;
     int const hf = lane & 1;
-    int64_t const tRaw = (int64_t) blockIdx.x * TOK + tok;
+    int64_t const tRaw = (int64_t) token_block_of_workgroup(blockIdx.x, gridDim.x) * TOK + tok;
     bool const valid = tRaw < total;
     // lanes past the last token re-read the last token (and store nothing): no divergent loads
     int64_t const t = valid ? tRaw : (int64_t) total - 1;
