@@ -299,7 +299,7 @@ def run_encoder(args, api, torch):
             "hbm_frac": round(4 * T * E / (table["attention"]["avg_launch_us"] * 1e-6) / PEAK_HBM, 4),
         },
         "roofline_skipln": {
-            "kernel": "skipln_interleaved_kernel<32,8,32,false>",
+            "kernel": "skipln_interleaved_kernel<32,8,32,false,true>",
             "bound": "hbm",
             "achieved": table["skipln"]["GB/s"],
             "peak": PEAK_HBM / 1e9,
@@ -659,7 +659,7 @@ def main():
             "hbm_frac": round(wl.mha_bytes() / t_mha / PEAK_HBM, 4),
         },
         "roofline_skipln": {
-            "kernel": "skipln_interleaved_kernel<32,8,32,false>",
+            "kernel": "skipln_interleaved_kernel<32,8,32,false,false>",
             "bound": "hbm",
             "achieved": round(ln_bytes / t_ln / 1e9, 1),
             "peak": PEAK_HBM / 1e9,

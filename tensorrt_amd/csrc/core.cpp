@@ -40,6 +40,20 @@ void read_tuning_env()
 }
 } // namespace
 
+int num_cus()
+{
+    static int const n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess
+            || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        {
+            cus = 256;
+        }
+        return cus;
+    }();
+    return n;
+}
+
 int tuning(Tuning which)
 {
     std::call_once(gTuningOnce, read_tuning_env);

@@ -54,6 +54,9 @@ enum class Tuning : int
 };
 int tuning(Tuning which);
 
+// Compute units of the current device, asked once per process (256 when the query fails).
+int num_cus();
+
 template <typename T>
 constexpr T ceil_div(T a, T b)
 {

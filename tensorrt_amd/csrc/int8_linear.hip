@@ -1149,20 +1149,6 @@ __global__ __launch_bounds__(512) void int8_linear_dma_kernel(LinearArgs const p
     }
 }
 
-int num_cus()
-{
-    static int const n = [] {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess
-            || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-        {
-            cus = 256;
-        }
-        return cus;
-    }();
-    return n;
-}
-
 template <bool IL_W, bool IL_IN, bool IL_OUT, int EPI>
 int launch_shape(hipStream_t stream, LinearArgs a)
 {

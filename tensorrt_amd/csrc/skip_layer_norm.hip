@@ -432,7 +432,7 @@ __device__ inline uint32_t token_block_of_workgroup(uint32_t bid, uint32_t nbloc
     return first + (x % kXcds) * run + x / kXcds;
 }
 
-template <int G, int W, int TOK, bool PRELN>
+template <int G, int W, int TOK, bool PRELN, bool TAIL>
 __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int const total,
     int8_t const* __restrict__ in, int8_t const* __restrict__ skip, f16 const* __restrict__ beta,
     f16 const* __restrict__ gamma, int8_t* __restrict__ out, int8_t* __restrict__ preln, float const dqIn,
@@ -456,7 +456,8 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
     int const sub = lane / LPG;
     int const tok = (lane % LPG) >> 1;
     int const hf = lane & 1;
-    int64_t const tRaw = (int64_t) token_block_of_workgroup(blockIdx.x, gridDim.x) * TOK + tok;
+    uint32_t const block = token_block_of_workgroup(blockIdx.x, gridDim.x);
+    int64_t const tRaw = (int64_t) block * TOK + tok;
     bool const valid = tRaw < total;
     // lanes past the last token re-read the last token (and store nothing): no divergent loads
     int64_t const t = valid ? tRaw : (int64_t) total - 1;
@@ -471,6 +472,28 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
     {
         xi[i] = *reinterpret_cast<u32x4 const*>(in + base + i * kStep * groupStride);
         xs[i] = *reinterpret_cast<u32x4 const*>(skip + base + i * kStep * groupStride);
+    }
+    // TAIL: a launch of fewer workgroups than token blocks (launch_interleaved: token counts just above one round of
+    // resident workgroups) leaves tokens behind the last block, and workgroup b also takes token gridDim.x * TOK + b.
+    // Its first wavefront requests that token's two rows now, straight into LDS (lane = channel group x half; no
+    // vector registers held), and normalises it after the block.
+    constexpr int kExtraLoads = (G + 31) / 32; // load instructions per tensor: 32 channel groups x 2 halves each
+    __shared__ __attribute__((aligned(16))) uint8_t sExtra[2][TAIL ? kExtraLoads * 1024 : 16];
+    int64_t const extraTok = (int64_t) gridDim.x * TOK + block;
+    bool const hasExtra = TAIL && extraTok < total; // the same for every lane of the workgroup
+    if (TAIL && hasExtra && wave == 0)
+    {
+#pragma unroll
+        for (int e = 0; e < kExtraLoads; ++e)
+        {
+            int const grp = e * 32 + (lane >> 1);
+            if (grp < G)
+            {
+                int64_t const off = (int64_t) grp * groupStride + extraTok * 32 + hf * 16;
+                load_to_lds16(in + off, (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) sExtra[0] + e * 1024);
+                load_to_lds16(skip + off, (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) sExtra[1] + e * 1024);
+            }
+        }
     }
     // gamma/beta are staged after the tensor loads were issued, so their latency overlaps
     for (int i = threadIdx.x; i < LD; i += THREADS)
@@ -523,6 +546,12 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
             sStat[wave][tok][3] = sIS;
             sStat[wave][tok][4] = sSS;
         }
+    }
+    if (TAIL && hasExtra && wave == 0)
+    {
+        // the block's rows have arrived (the statistics above consumed them), and so have the extra token's, requested
+        // right behind them: this wait makes that explicit for loads the compiler does not see, and costs nothing here
+        wait_vmcnt<0>();
     }
     __syncthreads();
     if (W > 1)
@@ -595,6 +624,134 @@ __global__ __launch_bounds__(W * kWaveSize) void skipln_interleaved_kernel(int c
             }
         }
     }
+    if constexpr (TAIL)
+    if (hasExtra && wave == 0)
+    {
+        // The extra token, once the block's registers are free: its rows have been in LDS since before the barrier.
+        // Lane = (channel group, half) as it loaded; the whole wavefront is one token.
+        int eIn = 0, eSk = 0, eII = 0, eIS = 0, eSS = 0;
+        u32x4 ea[kExtraLoads], es[kExtraLoads];
+#pragma unroll
+        for (int e = 0; e < kExtraLoads; ++e)
+        {
+            bool const live = e * 32 + (lane >> 1) < G;
+            ea[e] = live ? *reinterpret_cast<u32x4 const*>(sExtra[0] + e * 1024 + lane * 16) : u32x4{0, 0, 0, 0};
+            es[e] = live ? *reinterpret_cast<u32x4 const*>(sExtra[1] + e * 1024 + lane * 16) : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                eIn = __builtin_amdgcn_sdot4((int) ea[e][q], 0x01010101, eIn, false);
+                eSk = __builtin_amdgcn_sdot4((int) es[e][q], 0x01010101, eSk, false);
+                eII = __builtin_amdgcn_sdot4((int) ea[e][q], (int) ea[e][q], eII, false);
+                eIS = __builtin_amdgcn_sdot4((int) ea[e][q], (int) es[e][q], eIS, false);
+                eSS = __builtin_amdgcn_sdot4((int) es[e][q], (int) es[e][q], eSS, false);
+            }
+        }
+        eIn = wave_sum_i32(eIn);
+        eSk = wave_sum_i32(eSk);
+        eII = wave_sum_i32(eII);
+        eIS = wave_sum_i32(eIS);
+        eSS = wave_sum_i32(eSS);
+        // the two scales converted again from copies the compiler takes as new: kept from the block's statistics,
+        // the binary64 values would hold four vector registers through the block's arithmetic and cost the kernel a
+        // resident workgroup per CU
+        float dqI = dqIn, dqS = dqSkip;
+        asm volatile("" : "+s"(dqI), "+s"(dqS));
+        double const xIn = (double) dqI, xSk = (double) dqS;
+        double const eMean = (xIn * eIn + xSk * eSk) * (1.0 / LD);
+        double const eEx2 = (xIn * xIn * eII + 2.0 * xIn * xSk * eIS + xSk * xSk * eSS) * (1.0 / LD);
+        float const eRsigma = rsqrtf(fmaxf((float) (eEx2 - eMean * eMean), 0.f) + eps);
+        float const e1 = dqI * eRsigma;
+        float const e2 = dqS * eRsigma;
+        float const ec = (float) (-eMean * (double) eRsigma);
+#pragma unroll
+        for (int e = 0; e < kExtraLoads; ++e)
+        {
+            int const grp = e * 32 + (lane >> 1);
+            int const ch = grp * 32 + hf * 16;
+            u32x4 o, po;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                uint32_t yw = 0, pw = 0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                {
+                    float const fa = i8_to_f32(ea[e][q], k);
+                    float const fs = i8_to_f32(es[e][q], k);
+                    float const nrm = fmaf(fa, e1, fmaf(fs, e2, ec));
+                    int const c = grp < G ? ch + q * 4 + k : 0;
+                    yw = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(sGamma[c], nrm, sBeta[c]), k, yw);
+                    if (PRELN)
+                    {
+                        float const pv = fmaf(fa, p1, fmaf(fs, p2, pc));
+                        pw = __builtin_amdgcn_cvt_pk_u8_f32(fmaxf(pv, prelnLo), k, pw);
+                    }
+                }
+                o[q] = yw ^ 0x80808080u;
+                if (PRELN)
+                {
+                    po[q] = pw ^ 0x80808080u;
+                }
+            }
+            if (grp < G)
+            {
+                int64_t const off = (int64_t) grp * groupStride + extraTok * 32 + hf * 16;
+                store_through_l2(out + off, o);
+                if (PRELN)
+                {
+                    store_through_l2(preln + off, po);
+                }
+            }
+        }
+    }
+}
+
+// Workgroups of this kernel that the current device holds at once (asked once per process and kernel; 0 when it
+// cannot be asked).
+template <int G, int W, int TOK, bool PRELN, bool TAIL>
+int resident_workgroups()
+{
+    static int const n = [] {
+        int perCu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                &perCu, skipln_interleaved_kernel<G, W, TOK, PRELN, TAIL>, W * kWaveSize, 0)
+                != hipSuccess
+            || perCu <= 0)
+        {
+            (void) hipGetLastError();
+            return 0;
+        }
+        return perCu * num_cus();
+    }();
+    return n;
+}
+
+template <int G, int W, int TOK, bool PRELN>
+int launch_interleaved_as(hipStream_t stream, int32_t total, int8_t const* in, int8_t const* skip, f16 const* beta,
+    f16 const* gamma, int8_t* out, int8_t* preln, float dqIn, float dqSkip, float qScale, float qSkipScale, float eps,
+    float prelnMin)
+{
+    // One workgroup per block of TOK tokens.  When that is a few workgroups more than the chip holds at once, the
+    // stragglers of a second round cost 1.4-1.7 us whatever their number (33280 tokens x 1024 channels: 18.7 us where
+    // 32736 tokens take 17.0), so when one token more per workgroup lets a single round cover the tensor the launch is
+    // that round, with the kernel's tail path.
+    int const blocks = ceil_div(total, TOK);
+    dim3 const block(W * kWaveSize);
+    int const residentPlain = resident_workgroups<G, W, TOK, PRELN, false>();
+    int const residentTail = resident_workgroups<G, W, TOK, PRELN, true>();
+    if (residentPlain > 0 && blocks > residentPlain && residentTail > 0 && residentTail < blocks
+        && (int64_t) residentTail * (TOK + 1) >= total)
+    {
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, PRELN, true>), dim3((unsigned) residentTail), block, 0,
+            stream, total, in, skip, beta, gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
+    }
+    else
+    {
+        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, PRELN, false>), dim3((unsigned) blocks), block, 0, stream,
+            total, in, skip, beta, gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
+    }
+    return check_launch("skipln_interleaved_kernel");
 }
 
 template <int G, int W, int TOK>
@@ -602,19 +759,10 @@ int launch_interleaved(hipStream_t stream, int32_t total, int8_t const* in, int8
     f16 const* gamma, int8_t* out, int8_t* preln, float dqIn, float dqSkip, float qScale, float qSkipScale, float eps,
     float prelnMin)
 {
-    dim3 const grid((unsigned) ceil_div(total, TOK));
-    dim3 const block(W * kWaveSize);
-    if (preln)
-    {
-        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, true>), grid, block, 0, stream, total, in, skip, beta,
-            gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
-    }
-    else
-    {
-        hipLaunchKernelGGL((skipln_interleaved_kernel<G, W, TOK, false>), grid, block, 0, stream, total, in, skip, beta,
-            gamma, out, preln, dqIn, dqSkip, qScale, qSkipScale, eps, prelnMin);
-    }
-    return check_launch("skipln_interleaved_kernel");
+    return preln ? launch_interleaved_as<G, W, TOK, true>(stream, total, in, skip, beta, gamma, out, preln, dqIn, dqSkip,
+               qScale, qSkipScale, eps, prelnMin)
+                 : launch_interleaved_as<G, W, TOK, false>(stream, total, in, skip, beta, gamma, out, preln, dqIn, dqSkip,
+                     qScale, qSkipScale, eps, prelnMin);
 }
 
 // small: epsilon = binary16 epsilon, preln clipped to +-127; large: binary32 epsilon, preln

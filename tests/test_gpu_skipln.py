@@ -176,6 +176,18 @@ def test_skipln_interleaved(api, variant, large, ld, total):
                           max_frac_off=0.01)
 
 
+@pytest.mark.parametrize("variant,large,ld,total", [
+    # token counts just above what one round of resident workgroups covers in blocks of 32 tokens (256 CUs x 4, x 2,
+    # x 5 workgroups): the launch then is that one round, each workgroup taking one token more (the kernel's tail
+    # path), up to 33 tokens per workgroup; one count beyond, one far beyond
+    (0, True, 1024, 32769), (0, True, 1024, 33289), (0, True, 1024, 33792), (0, True, 1024, 33793),
+    (1, True, 1024, 16385), (1, True, 1024, 16896), (1, False, 1024, 16700), (0, True, 768, 40999),
+    (1, False, 2048, 16500), (1, False, 4096, 8300), (0, False, 768, 33000),
+])
+def test_skipln_interleaved_one_round_with_tail(api, variant, large, ld, total):
+    test_skipln_interleaved(api, variant, large, ld, total)
+
+
 def test_skipln_interleaved_saturation(api):
     """preln: the small kernel clips to -127, the large one saturates to -128."""
     ld, total = 1024, 8
