@@ -188,6 +188,32 @@ def test_skipln_interleaved_one_round_with_tail(api, variant, large, ld, total):
     test_skipln_interleaved(api, variant, large, ld, total)
 
 
+def test_skipln_interleaved_tail_launch_replays_from_a_graph(api):
+    """The one-round launch (its workgroup count comes from an occupancy query, its extra tokens travel through LDS)
+    recorded in a graph: every replay gives the eager bytes."""
+    import torch
+    ld, total = 1024, 33001
+    r = rng(31)
+    x, s, dq_in, dq_skip = _int8_inputs(r, total, ld)
+    gamma, beta, _ = _ln_params(r, ld, np.float16)
+    q_scale = np.float32(127.0 / 4.5)
+    dx, ds, db, dg = dev(oracle.interleave(x)), dev(oracle.interleave(s)), dev(beta), dev(gamma)
+    eager, replayed = dev_empty((ld * total,), np.int8, fill=0), dev_empty((ld * total,), np.int8, fill=0)
+    api.check(api.skipln_interleaved_large_hface(stream(), ld, total, ptr(dx), ptr(ds), ptr(db), ptr(dg), ptr(eager),
+                                                 dq_in, dq_skip, q_scale))
+    sync()
+    graph, cap = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.graph(graph, stream=cap):
+        api.check(api.skipln_interleaved_large_hface(cap.cuda_stream, ld, total, ptr(dx), ptr(ds), ptr(db), ptr(dg),
+                                                     ptr(replayed), dq_in, dq_skip, q_scale))
+    for _ in range(3):
+        replayed.zero_()
+        sync()
+        graph.replay()
+        sync()
+        assert np.array_equal(host(replayed), host(eager))
+
+
 def test_skipln_interleaved_saturation(api):
     """preln: the small kernel clips to -127, the large one saturates to -128."""
     ld, total = 1024, 8
