@@ -182,7 +182,8 @@ def test_skipln_interleaved(api, variant, large, ld, total):
     # path), up to 33 tokens per workgroup; one count beyond, one far beyond
     (0, True, 1024, 32769), (0, True, 1024, 33289), (0, True, 1024, 33792), (0, True, 1024, 33793),
     (1, True, 1024, 16385), (1, True, 1024, 16896), (1, False, 1024, 16700), (0, True, 768, 40999),
-    (1, False, 2048, 16500), (1, False, 4096, 8300), (0, False, 768, 33000),
+    (1, False, 2048, 16500), (1, False, 4096, 8300), (0, False, 768, 33000), (1, False, 1536, 16600),
+    (1, False, 3072, 8200), (1, True, 1024, 24577),
 ])
 def test_skipln_interleaved_one_round_with_tail(api, variant, large, ld, total):
     test_skipln_interleaved(api, variant, large, ld, total)
