@@ -99,6 +99,32 @@ __device__ inline void rows_transpose(uint32_t (&x)[4])
     x[3] = t23[1];
 }
 
+// Which unit of work ((sequence in serving order, head): unit / N, unit % N) and which part of its query tiles a
+// workgroup takes when qSplit workgroups share a unit.  Workgroup ids are dealt round-robin to the 8 XCDs, so ids
+// 8 q m + 8 p + x take unit 8 m + x, part p: the parts of a unit sit on one XCD and find its K and V in that L2, and
+// units are still started in id order, which is what serving the longest sequences first relies on (a renumbering
+// that gives each XCD one contiguous range of units starts the short sequences of the far end first: 80.7 against
+// 60.5 us for the encoder's launch at two workgroups per unit).  Ids behind the last whole span of 8 q keep the plain order.
+struct UnitPart
+{
+    uint32_t unit;
+    int part;
+};
+
+__device__ inline UnitPart unit_of_workgroup(uint32_t bid, uint32_t nblocks, int qSplit)
+{
+    if (qSplit <= 1)
+    {
+        return {bid, 0};
+    }
+    uint32_t const q = (uint32_t) qSplit, span = 8u * q, m = bid / span, x = bid % span;
+    if ((m + 1) * span <= nblocks)
+    {
+        return {m * 8u + x % 8u, (int) (x / 8u)};
+    }
+    return {bid / q, (int) (bid % q)};
+}
+
 struct FmhaArgs
 {
     void const* qkv;
@@ -378,12 +404,10 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
     constexpr int kRow = Lds<1>::kRow;
 
     __shared__ int sLens[kMaxRanked + 1];
-    // workgroup ids are dealt round-robin to the 8 XCDs: when a head is split over several
-    // workgroups, renumber so that they land on one XCD and share K/V in its L2
-    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
-    int const part = bid % a.qSplit;
-    int const n = (bid / a.qSplit) % a.N;
-    int const b = pick_sequence<kWavesI8 * kWaveSize>(a, bid / (a.qSplit * a.N), sLens);
+    UnitPart const up = unit_of_workgroup(blockIdx.x, gridDim.x, a.qSplit);
+    int const part = up.part;
+    int const n = up.unit % a.N;
+    int const b = pick_sequence<kWavesI8 * kWaveSize>(a, up.unit / a.N, sLens);
     SeqInfo const sq = seq_info(a, b, KT * 64);
     int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
     if (part * kWavesI8 >= nqt)
@@ -1047,11 +1071,11 @@ __global__ __launch_bounds__(kWavesI8* kWaveSize) __attribute__((amdgpu_waves_pe
     uint8_t* sK = smem;
     uint8_t* sV = smem + Lds<1>::matBytes(KT);
     __shared__ PickLds sPick;
-    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
-    int const part = bid % a.qSplit;
-    int const n = (bid / a.qSplit) % a.N;
+    UnitPart const up = unit_of_workgroup(blockIdx.x, gridDim.x, a.qSplit);
+    int const part = up.part;
+    int const n = up.unit % a.N;
     int b;
-    SeqInfo const sq = pick_sequence_info<kWavesI8 * kWaveSize>(a, bid / (a.qSplit * a.N), KT * 64, sPick, b);
+    SeqInfo const sq = pick_sequence_info<kWavesI8 * kWaveSize>(a, up.unit / a.N, KT * 64, sPick, b);
     // contiguous tile ranges, each a multiple of one round of the workgroup's wavefronts
     int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
     int const per = kWavesI8 * ((nqt + kWavesI8 * a.qSplit - 1) / (kWavesI8 * a.qSplit));
@@ -1115,12 +1139,10 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_kernel(FmhaArgs
     constexpr int kRow = Lds<2>::kRow;
 
     __shared__ int sLens[kMaxRanked + 1];
-    // workgroup ids are dealt round-robin to the 8 XCDs: when a head is split over several
-    // workgroups, renumber so that they land on one XCD and share K/V in its L2
-    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
-    int const part = bid % a.qSplit;
-    int const n = (bid / a.qSplit) % a.N;
-    int const b = pick_sequence<kWavesF16 * kWaveSize>(a, bid / (a.qSplit * a.N), sLens);
+    UnitPart const up = unit_of_workgroup(blockIdx.x, gridDim.x, a.qSplit);
+    int const part = up.part;
+    int const n = up.unit % a.N;
+    int const b = pick_sequence<kWavesF16 * kWaveSize>(a, up.unit / a.N, sLens);
     SeqInfo const sq = seq_info(a, b, KT * 64);
     int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
     if (part * kWavesF16 >= nqt)
@@ -1574,11 +1596,11 @@ __global__ __launch_bounds__(kWavesF16* kWaveSize) void fmha_f16_prefix_kernel(F
     uint8_t* sK = smem;
     uint8_t* sV = smem + Lds<2>::matBytes(KT);
     __shared__ PickLds sPick;
-    uint32_t const bid = a.qSplit > 1 ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
-    int const part = bid % a.qSplit;
-    int const n = (bid / a.qSplit) % a.N;
+    UnitPart const up = unit_of_workgroup(blockIdx.x, gridDim.x, a.qSplit);
+    int const part = up.part;
+    int const n = up.unit % a.N;
     int b;
-    SeqInfo const sq = pick_sequence_info<kWavesF16 * kWaveSize>(a, bid / (a.qSplit * a.N), KT * 64, sPick, b);
+    SeqInfo const sq = pick_sequence_info<kWavesF16 * kWaveSize>(a, up.unit / a.N, KT * 64, sPick, b);
     int const nqt = (sq.nq + kQPerWave - 1) / kQPerWave;
     int const per = kWavesF16 * ((nqt + kWavesF16 * a.qSplit - 1) / (kWavesF16 * a.qSplit));
     int const qtBegin = min(part * per, nqt);
@@ -1862,18 +1884,28 @@ int fused_mha_run(hipStream_t stream, int32_t dataType, trtamd_fmha_params const
     a.N = p->h;
     a.S = p->s;
     {
-        // Workgroups per (sequence, head): one, unless the launch would leave compute units idle.
-        // Every extra workgroup stages K and V again, which costs more than it gains once the
-        // chip is full, so heads are only shared while there are fewer of them than workgroup slots
-        // worth filling (one per CU for FP16, whose K/V take most of a CU's LDS; two for INT8).
+        // Workgroups per (sequence, head).  Every extra workgroup stages K and V again, so a unit is only shared
+        // while the launch would otherwise leave the chip partly idle or badly balanced.  INT8 (three workgroups per
+        // CU, 768 places): below 896 units two workgroups per unit, which also evens out a single round of units of
+        // very different lengths (768 units of 128-384 keys: 24.9 against 27.8 us; 512 units: 18.7 against 23.1 us;
+        // 896 units: 29.1 against 28.1 us), and more of them only to reach one round (256 units: three, 12.6 us
+        // against 13.1 with two and 17.4 with one; at most four).  FP16 (its K and V take most of a CU's LDS, one
+        // workgroup per CU, and staging them is 40 % of a workgroup's time): only below 160 units (192 units of 192-384
+        // keys: 15.3 us alone, 17.5 us shared by two; 144 units: 14.9 against 12.9 us).
         int const waves = dataType == 2 ? kWavesI8 : kWavesF16;
         int const maxSplit = std::max(1, ceil_div(ceil_div(p->s, kQPerWave), waves));
         int64_t const heads = (int64_t) p->b * p->h;
-        int64_t const target = dataType == 2 ? 512 : 256;
         int split = 1;
-        while (split < maxSplit && heads * split < target)
+        if (dataType == 2)
         {
-            split *= 2;
+            split = heads >= 896 ? 1 : (int) std::max<int64_t>(2, std::min<int64_t>(4, ceil_div<int64_t>(768, heads)));
+        }
+        else
+        {
+            while (split < maxSplit && heads * split < 160)
+            {
+                split *= 2;
+            }
         }
         a.qSplit = std::min(split, maxSplit);
         // tuning override: TRTAMD_FMHA_QSPLIT=<n> forces the number of workgroups per head

@@ -86,7 +86,8 @@ def test_linear_variants(name, value, il):
 
 
 FMHA_SETTINGS = [("TRTAMD_FMHA_GENERIC", 1), ("TRTAMD_FMHA_QSPLIT", 1), ("TRTAMD_FMHA_QSPLIT", 2),
-                 ("TRTAMD_FMHA_QSPLIT", 4), ("TRTAMD_FMHA_RANKED", 0), ("TRTAMD_FMHA_RANKED", 1)]
+                 ("TRTAMD_FMHA_QSPLIT", 3), ("TRTAMD_FMHA_QSPLIT", 4), ("TRTAMD_FMHA_RANKED", 0),
+                 ("TRTAMD_FMHA_RANKED", 1)]
 
 
 @pytest.mark.parametrize("name,value", FMHA_SETTINGS)
