@@ -53,6 +53,9 @@ INT8_PACKED = [
     # B, N, S (max), lens rule
     (3, 2, 128, "rand"), (2, 16, 384, "c4"), (5, 3, 64, "rand"), (4, 2, 192, "rand"), (3, 2, 256, "full"),
     (2, 2, 512, "rand"), (6, 1, 96, "edge"),
+    # unit counts either side of where the launcher stops sharing a (sequence, head) unit between workgroups (896),
+    # a count that takes three workgroups per unit, and one whose ids do not fill whole spans of 8 x parts
+    (55, 16, 128, "rand"), (56, 16, 128, "rand"), (17, 16, 256, "c4"), (13, 3, 384, "rand"),
 ]
 
 
@@ -182,7 +185,9 @@ def test_fmha_fixed_nonprefix_mask(api):
 
 
 @pytest.mark.parametrize("B,N,S,rule", [(4, 12, 128, "c4"), (3, 12, 384, "c4"), (8, 2, 96, "edge"), (2, 16, 512, "rand"),
-                                        (3, 3, 192, "rand"), (2, 2, 256, "full")])
+                                        (3, 3, 192, "rand"), (2, 2, 256, "full"),
+                                        # either side of the unit count below which units are shared (160)
+                                        (13, 12, 192, "rand"), (14, 12, 192, "rand")])
 def test_fmha_fp16_packed(api, B, N, S, rule):
     from tensorrt_amd import capi
     r = rng(24)
