@@ -99,32 +99,6 @@ __device__ inline void rows_transpose(uint32_t (&x)[4])
     x[3] = t23[1];
 }
 
-// Which unit of work ((sequence in serving order, head): unit / N, unit % N) and which part of its query tiles a
-// workgroup takes when qSplit workgroups share a unit.  Workgroup ids are dealt round-robin to the 8 XCDs, so ids
-// 8 q m + 8 p + x take unit 8 m + x, part p: the parts of a unit sit on one XCD and find its K and V in that L2, and
-// units are still started in id order, which is what serving the longest sequences first relies on (a renumbering
-// that gives each XCD one contiguous range of units starts the short sequences of the far end first: 80.7 against
-// 60.5 us for the encoder's launch at two workgroups per unit).  Ids behind the last whole span of 8 q keep the plain order.
-struct UnitPart
-{
-    uint32_t unit;
-    int part;
-};
-
-__device__ inline UnitPart unit_of_workgroup(uint32_t bid, uint32_t nblocks, int qSplit)
-{
-    if (qSplit <= 1)
-    {
-        return {bid, 0};
-    }
-    uint32_t const q = (uint32_t) qSplit, span = 8u * q, m = bid / span, x = bid % span;
-    if ((m + 1) * span <= nblocks)
-    {
-        return {m * 8u + x % 8u, (int) (x / 8u)};
-    }
-    return {bid / q, (int) (bid % q)};
-}
-
 struct FmhaArgs
 {
     void const* qkv;
