@@ -198,15 +198,24 @@ def run_encoder(args, api, torch):
             with torch.cuda.graph(graph, stream=cap):
                 for _ in range(reps):
                     fn()
+            run = graph.replay
+        except RuntimeError:
+            # a measurement harness must not die on the recording: time the launches as they are issued instead
+            enc.stream = own
+            torch.cuda.synchronize()
+
+            def run():
+                for _ in range(reps):
+                    fn()
         finally:
             enc.stream = own
-        graph.replay()
+        run()
         torch.cuda.synchronize()
         best = None
         for _ in range(3):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            graph.replay()
+            run()
             e1.record()
             torch.cuda.synchronize()
             t = e0.elapsed_time(e1) * 1e-3 / reps
