@@ -462,6 +462,20 @@ def extra_rows(api, torch, steps: int = 100) -> list:
         rows.append({"kernel": f"INT8 linear {name} {Tq}x{K}x{Nn}", "gpu_us": round(t * 1e6, 2),
                      "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s", "frac": round(ops / t / PEAK_I8, 4)})
         del a8, w8, o8
+        # the vendor library on the same product (hipBLASLt behind torch._int_mm: row-major operands, INT32 output
+        # and no epilogue, so four times the output bytes and none of the requantisation); a comparison, not a leg
+        # of any workload
+        if epi == capi.LINEAR_AFFINE and hasattr(torch, "_int_mm"):
+            Tp = (Tq + 7) // 8 * 8   # _int_mm wants a multiple of 8 rows
+            A, Wt = qnormal((Tp, K)), qnormal((Nn, K)).t()
+            try:
+                t = timeit(lambda: torch._int_mm(A, Wt))
+                ops = 2.0 * Tp * K * Nn
+                rows.append({"kernel": f"  vendor library, torch._int_mm {Tp}x{K}x{Nn}, INT32 output", "gpu_us": round(t * 1e6, 2),
+                             "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s", "frac": round(ops / t / PEAK_I8, 4)})
+            except RuntimeError:
+                pass   # not every build of torch has the INT8 product
+            del A, Wt
     Th = 16384
     for name, K, Nn, epi in (("feed-forward 1 + GELU", 768, 3072, capi.LINEAR_GELU),
                              ("feed-forward 2", 3072, 768, capi.LINEAR_AFFINE)):
@@ -477,6 +491,11 @@ def extra_rows(api, torch, steps: int = 100) -> list:
         ops = 2.0 * Th * K * Nn
         rows.append({"kernel": f"FP16 linear {name} {Th}x{K}x{Nn}", "gpu_us": round(t * 1e6, 2),
                      "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s", "frac": round(ops / t / PEAK_F16, 4)})
+        if epi == capi.LINEAR_AFFINE:
+            bh = torch.zeros(Nn, dtype=torch.float16, device="cuda")
+            t = timeit(lambda: torch.nn.functional.linear(ah, wh, bh))
+            rows.append({"kernel": f"  vendor library, torch linear {Th}x{K}x{Nn}, FP16 + bias", "gpu_us": round(t * 1e6, 2),
+                         "achieved": round(ops / t / 1e12, 1), "unit": "TOP/s", "frac": round(ops / t / PEAK_F16, 4)})
         del ah, wh, oh
     xh = torch.randn((Tq, 1024), dtype=torch.float16, device="cuda")
     x8 = torch.empty((32, Tq, 32), dtype=torch.int8, device="cuda")
